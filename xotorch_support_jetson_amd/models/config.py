@@ -100,12 +100,45 @@ class FeedForwardSpec:
   """A non-gated feed-forward W_down act(W_up h).  kind "polynorm": act(z) = a N(z) + b N(z^2) + c N(z^3) + e with N the
   division of the token's ff vector by its RMS; kind "relu2_moe": `experts` experts with act = relu^2, the `top` largest
   router logits chosen per token and weighted by the softmax over the chosen logits, plus (shared_ff > 0) one shared
-  expert of the same form scaled by a per-token sigmoid gate."""
-  kind: str  # polynorm | relu2_moe
+  expert of the same form scaled by a per-token sigmoid gate.
+  Gated kinds, W_down (a(W_gate h) * b(W_up h)): "clamped_glu": g = min(gate, limit), u = clamp(up, -limit, limit),
+  g sigmoid(1.702 g) (u + 1); "silu_moe": `experts` SiLU-gated experts, scores = softmax of the router logits over
+  all experts, the `top` largest chosen and weighted by their scores as they are (no renormalisation), plus
+  (shared_ff > 0) one ungated shared expert of the same form."""
+  kind: str  # polynorm | relu2_moe | clamped_glu | silu_moe
   ff: int
   experts: int = 0
   top: int = 0
   shared_ff: int = 0
+  limit: float = 0.0  # clamped_glu
+
+
+@dataclass(frozen=True)
+class LatentAttnSpec:
+  """Softmax attention through a low-rank key / value latent: per token the cache holds one RMS-normed latent c
+  [kv_rank] and one rotated key part [rot_dim] shared by every head.  Head h scores q_h = [dim unrotated | rot_dim
+  rotated] against [W_uk,h c | rotated part] (times scale) and sums the values W_uv,h c.  q_rank > 0: the queries go
+  through their own RMS-normed latent.  RoPE on the first rot_dims of the rot_dim part, pairs (2i, 2i + 1)
+  (rot_interleaved) or (i, i + rot_dims / 2).  window > 0: a query at position i sees 0 <= i - j < window, else every
+  j <= i.  sink: one learned logit per head joins the softmax's denominator (no key, no value, unscaled).  gate: the
+  heads' outputs times sigmoid of a projection of the mixer's input, per element ("elem") or per head ("head")."""
+  heads: int
+  dim: int
+  rot_dim: int
+  vdim: int
+  kv_rank: int
+  q_rank: int
+  rot_dims: int
+  rot_base: float
+  rot_interleaved: bool
+  scale: float
+  window: int = 0
+  sink: bool = False
+  gate: str = "none"  # none | elem | head
+
+  @property
+  def gate_rows(self) -> int:
+    return {"none": 0, "elem": self.heads * self.vdim, "head": self.heads}[self.gate]
 
 
 @dataclass(frozen=True)
@@ -123,10 +156,14 @@ class MixedLayerSpec:
   wattn: Optional[WindowAttnSpec] = None
   ssd: Optional[SSDSpec] = None
   ffn: Optional[FeedForwardSpec] = None
+  lattn: Optional[LatentAttnSpec] = None  # sandwich blocks
 
   @property
   def kv_dims(self) -> Optional[tuple]:
-    """(kv heads, key dim, value dim) of the paged K / V pool this layer owns (None: it has none of its own)."""
+    """(kv heads, key dim, value dim) of the paged K / V pool this layer owns (None: it has none of its own).  A
+    latent-attention layer keeps one row [kv_rank | rot_dim] per token and no value pool (value dim 0)."""
+    if self.lattn is not None:
+      return 1, self.lattn.kv_rank + self.lattn.rot_dim, 0
     if self.attn is not None:
       return self.attn.kv_heads, self.attn.dim, self.attn.dim
     if self.wattn is not None and self.wattn.kv_from < 0:
@@ -147,7 +184,7 @@ class MixedLayerSpec:
 
 @dataclass(frozen=True)
 class ModelConfig:
-  model_type: str  # llama | qwen2 | mistral | mixtral | ... | tarepel | mogelix
+  model_type: str  # llama | qwen2 | mistral | mixtral | ... | tarepel | mogelix | nenizen
   vocab_size: int
   hidden_size: int
   intermediate_size: int
@@ -199,6 +236,28 @@ class ModelConfig:
   # (Mogelix: x <- norm(alpha x + gate * sublayer(x)) for the mixer, then for the feed-forward; per-channel norm weights)
   block: str = "parallel"
   postln_alpha: float = 1.0
+  # "sandwich" blocks (Nenizen): x += norm_b(mixer(norm(x))), then x += norm_b(ff(norm(x))), per-channel weights.
+  # loop = (start, stop, times): layers start .. stop - 1 run `times` times in a row with the same weights and a cache
+  # of their own per pass; each pass starts with x <- W_in [x; embedding output] + step[pass]
+  embed_scale: float = 1.0
+  logit_softcap: float = 0.0  # > 0: logits <- cap * tanh(logits / cap)
+  loop: Optional[tuple] = None
+
+  def layer_runs(self, layers=None) -> list:
+    """[(layer, pass or -1)] in execution order for the given layers (default: all): a looped layer appears once per
+    pass; pass >= 0 marks the first layer of a pass (where the pass's input mix happens)."""
+    ids = list(range(self.num_layers)) if layers is None else list(layers)
+    if not self.loop:
+      return [(i, -1) for i in ids]
+    a, b, times = self.loop
+    inside = [i for i in ids if a <= i < b]
+    if inside and (inside != list(range(a, b)) or ids[0] != 0):
+      raise ValueError(f"layers {a}..{b - 1} run as a loop that mixes in the embedding output: a shard must hold all of "
+                       "them together with the first layer")
+    out = [(i, -1) for i in ids if i < a]
+    for t in range(times if inside else 0):
+      out += [(i, t if i == a else -1) for i in inside]
+    return out + [(i, -1) for i in ids if i >= b]
 
   @property
   def is_mixed(self) -> bool:
@@ -295,6 +354,17 @@ class ModelConfig:
 
 
 def mixed_layer_params(D: int, s: MixedLayerSpec) -> int:
+  if s.lattn is not None:
+    a, f = s.lattn, s.ffn
+    qd = a.heads * (a.dim + a.rot_dim)
+    n = 4 * D + (D * a.q_rank + a.q_rank + a.q_rank * qd if a.q_rank else D * qd)
+    n += D * (a.kv_rank + a.rot_dim) + a.kv_rank + a.kv_rank * a.heads * (a.dim + a.vdim) + a.heads * a.vdim * D
+    n += a.gate_rows * D + (a.heads if a.sink else 0)
+    if f is not None and f.kind == "clamped_glu":
+      n += 3 * D * f.ff
+    elif f is not None:
+      n += f.experts * (3 * D * f.ff + D) + 3 * D * f.shared_ff
+    return n
   if s.wattn is not None or s.ssd is not None:
     n = 2 * D * (D + 1) + 2 * D  # the two sublayer gates and norms
     if s.wattn is not None:
@@ -444,7 +514,67 @@ def _mogelix_config(cfg: dict) -> ModelConfig:
     layer_specs=tuple(specs), block="postln", postln_alpha=float(cfg.get("postln_alpha", 1.0)))
 
 
+_LATENT_KINDS = {
+  # layer type: (queries through a latent, interleaved rotation pairs, sliding window, sink, output gate)
+  "latent_attention": (False, True, False, False, "elem"),
+  "latent_attention_2": (True, False, True, False, "head"),
+  "latent_attention_3": (True, False, False, True, "none"),
+}
+
+
+def _nenizen_config(cfg: dict) -> ModelConfig:
+  """Nenizen config.json: {"architecture", "vocab", "width", "norm": {"eps"}, "embedding": {"scale"}, "logit_softcap",
+  "loop": {"start", "stop", "times"} | null, "layers": [{"type": "latent_attention" | "latent_attention_2" |
+  "latent_attention_3", "mixer": {"heads", "dim", "rot_dim", "vdim", "kv_rank", "q_rank", "rot": {"base", "dims"},
+  "scale", "mask": {"size"}}, "mlp": {"kind": "dense", "ff", "limit"} | {"kind": "moe", "expert": {"ff"}, "router":
+  {"experts", "top"}, "shared": {"ff"}} | null}]}."""
+  specs = []
+  for i, L in enumerate(cfg["layers"]):
+    m, mlp = L["mixer"], L.get("mlp")
+    if L["type"] not in _LATENT_KINDS:
+      raise ValueError(f"layer {i}: unknown layer type {L['type']!r}")
+    qlat, inter, windowed, sink, gate = _LATENT_KINDS[L["type"]]
+    rot = m.get("rot") or {}
+    a = LatentAttnSpec(int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                       int(m["q_rank"]) if qlat else 0, int(rot.get("dims", 0)), float(rot.get("base", 10000.0)), inter,
+                       float(m["scale"]), int(m["mask"]["size"]) if windowed else 0, sink, gate)
+    if a.rot_dims % 2 or a.rot_dims > a.rot_dim or min(a.heads, a.dim + a.rot_dim, a.vdim, a.kv_rank) < 1 or \
+       (windowed and a.window < 1):
+      raise ValueError(f"layer {i}: sizes of the latent attention do not fit")
+    ffn = None
+    if mlp is not None:
+      kind = mlp.get("kind", "dense")
+      if kind == "dense":
+        ffn = FeedForwardSpec("clamped_glu", int(mlp["ff"]), limit=float(mlp["limit"]))
+      elif kind == "moe":
+        sh = mlp.get("shared")
+        ffn = FeedForwardSpec("silu_moe", int(mlp["expert"]["ff"]), int(mlp["router"]["experts"]),
+                              int(mlp["router"]["top"]), int(sh["ff"]) if sh else 0)
+        if not 1 <= ffn.top <= ffn.experts:
+          raise ValueError(f"layer {i}: top {ffn.top} of {ffn.experts} experts")
+      else:
+        raise ValueError(f"layer {i}: unsupported feed-forward kind {kind!r}")
+    specs.append(MixedLayerSpec(L["type"], lattn=a, ffn=ffn))
+  lp = cfg.get("loop")
+  loop = None
+  if lp and int(lp.get("times", 1)) >= 1 and int(lp["stop"]) > int(lp["start"]):
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+    if not 0 <= loop[0] < loop[1] <= len(specs):
+      raise ValueError(f"loop {loop} outside the {len(specs)} layers")
+  first = specs[0].lattn
+  return ModelConfig(
+    model_type="nenizen", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+    intermediate_size=max([s.ffn.ff for s in specs if s.ffn is not None] + [0]), num_layers=len(specs),
+    num_heads=first.heads, num_kv_heads=1, head_dim=first.dim + first.rot_dim, rms_norm_eps=float(cfg["norm"]["eps"]),
+    rope_theta=first.rot_base, max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
+    tie_word_embeddings=True, bos_token_id=int(cfg.get("bos_token_id", 0)), eos_token_ids=tuple(cfg.get("eos_token_ids", ())),
+    layer_specs=tuple(specs), block="sandwich", embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+    logit_softcap=float(cfg.get("logit_softcap") or 0.0), loop=loop)
+
+
 def from_hf_config(cfg: dict) -> ModelConfig:
+  if cfg.get("architecture") == "Nenizen":
+    return _nenizen_config(cfg)
   if cfg.get("architecture") == "Tarepel":
     return _tarepel_config(cfg)
   if cfg.get("architecture") == "Mogelix":
@@ -694,6 +824,28 @@ TINY_MOGELIX = {
      "mixer": {"heads": 2, "vdim": 32, "state": 16, "groups": 1, "conv": 4, "norm_groups": 1}},
   ]}
 PRESETS["tiny-mogelix"] = _mogelix_config(TINY_MOGELIX)
+_TINY_LMOE = {"kind": "moe", "expert": {"ff": 40}, "router": {"experts": 5, "top": 3}, "shared": {"ff": 24}}
+TINY_NENIZEN = {
+  "architecture": "Nenizen", "vocab": 272, "width": 80, "norm": {"eps": 1e-5}, "embedding": {"scale": 3.0},
+  "logit_softcap": 20.0, "loop": {"start": 1, "stop": 4, "times": 2},
+  "layers": [
+    {"type": "latent_attention_2", "mlp": {"kind": "dense", "ff": 112, "limit": 1.5},
+     "mixer": {"heads": 3, "dim": 24, "rot_dim": 8, "vdim": 20, "kv_rank": 48, "q_rank": 40, "mask": {"size": 11},
+               "rot": {"base": 10000.0, "dims": 8}, "scale": 0.2}},
+    {"type": "latent_attention", "mlp": _TINY_LMOE,
+     "mixer": {"heads": 5, "dim": 8, "rot_dim": 16, "vdim": 16, "kv_rank": 32,
+               "rot": {"base": 50000.0, "dims": 16}, "scale": 0.25}},
+    {"type": "latent_attention_3", "mlp": None,
+     "mixer": {"heads": 2, "dim": 16, "rot_dim": 16, "vdim": 40, "kv_rank": 24, "q_rank": 16,
+               "rot": {"base": 1000.0, "dims": 12}, "scale": 0.3}},
+    {"type": "latent_attention_2", "mlp": _TINY_LMOE,
+     "mixer": {"heads": 4, "dim": 16, "rot_dim": 4, "vdim": 8, "kv_rank": 64, "q_rank": 24, "mask": {"size": 70},
+               "rot": {"base": 10000.0, "dims": 4}, "scale": 0.2}},
+    {"type": "latent_attention_3", "mlp": {"kind": "dense", "ff": 96, "limit": 3.0},
+     "mixer": {"heads": 4, "dim": 16, "rot_dim": 16, "vdim": 16, "kv_rank": 32, "q_rank": 48,
+               "rot": {"base": 10000.0, "dims": 16}, "scale": 0.2}},
+  ]}
+PRESETS["tiny-nenizen"] = _nenizen_config(TINY_NENIZEN)
 # aliases of the reference's model cards that share an architecture
 for _alias, _base in {"llama-3.1-70b-bf16": "llama-3.1-70b", "nemotron-70b": "llama-3.1-70b",
                       "deepseek-r1-distill-llama-70b": "llama-3.1-70b", "deepseek-r1-distill-llama-8b": "llama-3.1-8b",

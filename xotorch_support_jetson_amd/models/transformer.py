@@ -97,10 +97,13 @@ class KVCache:
     if c.is_mixed:
       # one K [pages, G, 64, d] and one V [pages, G, d, 64] pool per layer that has an attention mixer (None for the others):
       # layers may differ in heads and sizes; the value pool holds whatever the layer's mixer stores as values
-      ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
+      # (one entry per layer RUN: a looped layer has a cache of its own in every pass, config.layer_runs)
+      ids = [i for i, _ in c.layer_runs(layer_ids if layer_ids is not None else range(n_layers))]
       dims = [c.layer_specs[i].kv_dims for i in ids]
       self.k = [None if a is None else torch.zeros(num_pages, a[0], PAGE, a[1], device=device, dtype=dtype) for a in dims]
-      self.v = [None if a is None else torch.zeros(num_pages, a[0], a[2], PAGE, device=device, dtype=dtype) for a in dims]
+      # (latent attention keeps no value pool: the cached latent is key and value, value dim 0)
+      self.v = [None if a is None or not a[2] else torch.zeros(num_pages, a[0], a[2], PAGE, device=device, dtype=dtype)
+                for a in dims]
       # window attention with pooled blocks: per layer the (source layer, block size) pooled caches it reads, K
       # [pages, G, per, d] and V [pages, G, per, dv]; entries live with the page of a block's last token, so they are
       # handed out and returned with the sequence's pages.  pool_owner[j]: this layer fills them (the first layer of
@@ -137,7 +140,7 @@ class KVCache:
   @staticmethod
   def bytes_per_page(c: ModelConfig, n_layers: int, layer_ids=None, itemsize: int = 2) -> int:
     if c.is_mixed:
-      ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
+      ids = [i for i, _ in c.layer_runs(layer_ids if layer_ids is not None else range(n_layers))]
       n, seen = 0, set()
       for i in ids:
         a, w = c.layer_specs[i].kv_dims, c.layer_specs[i].wattn
@@ -170,7 +173,7 @@ class StatePool:
     self.slots = slots
     self.S: List[Optional[torch.Tensor]] = []
     self.conv: List[Optional[torch.Tensor]] = []
-    for i in layer_ids:
+    for i, _ in c.layer_runs(layer_ids):  # (a looped layer: a state of its own in every pass)
       sd = c.layer_specs[i].state_dims  # (heads, value dim, key dim, taps, convolution channels)
       self.S.append(None if sd is None else torch.zeros(slots, sd[0], sd[1], sd[2], device=device, dtype=torch.float32))
       self.conv.append(torch.zeros(slots, max(sd[3] - 1, 0), sd[4], device=device, dtype=torch.float32)
@@ -212,6 +215,10 @@ class ShardModel:
                                       high_freq_factor=a.rot_scaling[2], original_max_position_embeddings=a.rot_scaling[3])
           self.rope_tabs[(a.rot_dims, a.rot_base, a.rot_scaling)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base,
                                                                                  sc, self.device)
+        a = c.layer_specs[i].lattn
+        if a is not None and a.rot_dims and (a.rot_dims, a.rot_base) not in self.rope_tabs:
+          self.rope_tabs[(a.rot_dims, a.rot_base)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base, None, self.device)
+      self.runs = c.layer_runs(self.layer_ids)
       return
     self.scale = 1.0 / math.sqrt(c.head_dim)
     max_pos = max(max_ctx, 16)
@@ -485,6 +492,8 @@ class ShardModel:
     adt = (w.layers[self.layer_ids[0]].in_w if n else w.lm_head).dtype
     if c.block == "postln":
       return self._forward_postln(h, inp, adt)
+    if c.block == "sandwich":
+      return self._forward_sandwich(h, inp, adt)
     bufs = {}
 
     def rows(name: str, live: int, padded: int) -> torch.Tensor:
@@ -667,6 +676,163 @@ class ShardModel:
     xn = torch.zeros(hl.shape[0], Dp, dtype=adt, device=h.device)
     K.gated_postnorm(hl, None, None, 0, None, 1.0, w.norm, c.rms_norm_eps, xn)
     return self._proj(xn, w.lm_head)[:, :c.vocab_size]
+
+  # ------------------------------------------------------------------ sandwich blocks (latent attention, gated feed-forwards)
+  def _latent_attn(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor, rows) -> None:
+    """Attention through the cached latent (one row [latent | rotated key part] per token): norms + RoPE + paged write,
+    the query up-projection (queries with a latent of their own), the unrotated query parts absorbed into the latent
+    space per head (q_lat = q W_uk), attention over the latent rows, the heads' values out of the latent space
+    (o = o_lat W_uv^T), the output gate."""
+    a, c, dev = lw.spec.lattn, self.c, P.device
+    T, adt = P.shape[0], mix.dtype
+    H, dn, dr, dv, R = a.heads, a.dim, a.rot_dim, a.vdim, a.kv_rank
+    tab = self.rope_tabs.get((a.rot_dims, a.rot_base))
+    rd = a.rot_dims if tab is not None else 0
+    tab = tab if tab is not None else torch.zeros(1, 0, device=dev)
+    qa = rows("qa", a.q_rank, lw.uq_w.shape[1]) if a.q_rank else None
+    K.latent_kv_store(P, lw.cols["ckv"][0], R, dr, lw.kv_norm, lw.cols["q"][0], a.q_rank, lw.q_norm, c.rms_norm_eps, rd,
+                      a.rot_interleaved, inp.positions, tab, inp.slots, self.kv.k[j], qa)
+    Q, q_off = (self._proj(qa, lw.uq_w), 0) if a.q_rank else (P, lw.cols["q"][0])
+    qn = torch.empty(H, T, dn, dtype=adt, device=dev)
+    qpe = torch.empty(T, H, dr, dtype=adt, device=dev)
+    K.latent_q_rope(Q, q_off, H, dn, dr, rd, a.rot_interleaved, inp.positions, tab, qn, qpe)
+    q_lat = self._bmm(qn, lw.uk_w)  # [H, T, R]
+    o_lat = torch.empty(H, T, R, dtype=adt, device=dev)
+    K.latent_attn(q_lat, qpe, self.kv.k[j], inp.block_tables, inp.cu_q, inp.ctx_lens, lw.sink, a.scale, a.window, o_lat,
+                  max_qlen=inp.max_qlen)
+    o = self._bmm(o_lat, lw.uv_w)  # [H, T, dv]
+    K.latent_out_gate(o, P, lw.cols["gate"][0] if a.gate != "none" else 0, {"none": 0, "elem": 1, "head": 2}[a.gate], mix)
+
+  @staticmethod
+  def _bmm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """Per-head products [H, T, k] x [H, k, n] on the vendor library (the CPU path multiplies in fp32)."""
+    if x.is_cuda:
+      return torch.bmm(x, w)
+    return torch.bmm(x.float(), w.float()).to(x.dtype)
+
+  def _silu_moe(self, hn: torch.Tensor, P: torch.Tensor, lw, rows) -> torch.Tensor:
+    """SiLU-gated experts chosen by the softmax scores' top-k (weights: the scores as they are) + the ungated shared
+    expert -> fp32 [T, D].  Routing on the framework's grouped top-k kernel, experts on the grouped GEMMs (bf16) or per
+    expert on the vendor SGEMM (fp32)."""
+    f, dev = lw.spec.ffn, P.device
+    T, D = hn.shape[0], self.c.hidden_size
+    E, k = f.experts, f.top
+    r0 = lw.ff_cols["router"][0]
+    logits = P[:, r0:r0 + E].contiguous()
+    Fp, Dq, S = lw.ex_down_w.shape[2], lw.ex_down_w.shape[1], 1
+    if P.is_cuda:
+      topw = torch.empty(T * k, dtype=torch.float32, device=dev)
+      topi, slot_of, sorted_tok = (torch.empty(T * k, dtype=torch.int32, device=dev) for _ in range(3))
+      off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+      K.moe_route_ds(logits, None, k, 1, 1, 0, False, False, 1.0, outs=(topw, topi, slot_of, sorted_tok, off))
+    else:
+      topw, idx = torch.topk(torch.softmax(logits.float(), -1), k, dim=-1)
+      topw, topi = topw.reshape(-1), idx.reshape(-1).int()
+      order = torch.argsort(topi, stable=True)
+      slot_of = torch.empty_like(order)
+      slot_of[order] = torch.arange(T * k)
+      sorted_tok = (order // k).int()
+      off = torch.cat([torch.zeros(1, dtype=torch.long), torch.bincount(topi.long(), minlength=E).cumsum(0)]).int()
+    if hn.dtype == torch.bfloat16 and hn.is_cuda:
+      C = require()
+      sh_up, sh_dn = layout_of(lw.ex_up_w) == "stream", layout_of(lw.ex_down_w) == "stream"
+      per_expert = T * k / E
+      big = sh_up and sh_dn and per_expert >= MOE_BIG_MIN_ROWS and Fp % 256 == 0 and Dq % 256 == 0
+      bm, bm_dn, S_dn = moe_tiles(per_expert, E) if big else (0, 0, 0)
+      if MOE_PP2:
+        bm, bm_dn = ({256: 2256, 192: 2192}.get(t, t) for t in (bm, bm_dn))
+      S = S_dn if big else (4 if T * k <= 64 else 2)
+      if Fp % (256 * S):
+        S = 1
+      gu = torch.empty(T * k, 2 * Fp, dtype=torch.float32, device=dev)
+      C.gemm_moe(hn, lw.ex_up_w, gu, off, sorted_tok, K.EPI["none"], T, sh_up, 1, bm)
+      act = torch.empty(T * k, Fp, dtype=torch.bfloat16, device=dev)
+      K.glu_act(gu, 0, Fp, Fp, False, 0.0, act)
+      y = torch.empty(S * T * k, Dq, dtype=torch.float32, device=dev)
+      C.gemm_moe(act, lw.ex_down_w, y, off, None, K.EPI["none"], T, sh_dn, S, bm_dn)
+    else:
+      # all-fp32 run (and the CPU path): one vendor SGEMM pair per expert that has rows (the offsets come to the host)
+      y = torch.zeros(T * k, Dq, dtype=torch.float32, device=dev)
+      offs = off.tolist()
+      for e in range(E):
+        if offs[e + 1] > offs[e]:
+          xe = hn.index_select(0, sorted_tok[offs[e]:offs[e + 1]].long()).float()
+          gu = xe @ lw.ex_up_w[e].float().t()
+          y[offs[e]:offs[e + 1]] = (torch.nn.functional.silu(gu[:, :Fp]) * gu[:, Fp:]) @ lw.ex_down_w[e].float().t()
+    sh_y = None
+    if f.shared_ff:
+      act = rows("sh_act", f.shared_ff, lw.down_w.shape[1])
+      K.glu_act(P, lw.ff_cols["sh_gate"][0], lw.ff_cols["sh_up"][0], f.shared_ff, False, 0.0, act)
+      sh_y = self._proj(act, lw.down_w)
+    out = torch.empty(T, D, dtype=torch.float32, device=dev)
+    K.moe_weighted_sum(y, slot_of, topw, k, sh_y, None, 0, out, splits=S)
+    return out
+
+  def _forward_sandwich(self, h: torch.Tensor, inp: StepInputs, adt) -> torch.Tensor:
+    """Layer runs (a looped layer once per pass, each pass with caches of its own) of sandwich blocks on the fp32
+    stream h (hn: the normed sublayer input in the GEMMs' operand dtype):
+      pass start:  h <- [h | embedding output] @ loop_in^T + step[pass]
+      P = hn @ in_w^T                    queries (or their latent), kv latent, rotated key part, output gate
+      h += norm1b(latent_attention(P) @ out_w^T);  hn = norm2(h)
+      P = hn @ ff_w^T                    gate | up, or router | shared gate | shared up
+      h += norm2b(ff(P));  hn = the next run's norm1(h)
+    Returns h (non-last shard) or softcap(head(final_norm(h rows inp.last_idx)))."""
+    c, w = self.c, self.w
+    T, D = h.shape
+    Dp = -(-D // 128) * 128
+    bufs = {}
+
+    def rows(name: str, live: int, padded: int) -> torch.Tensor:
+      key = (name, live, padded)
+      if key not in bufs:
+        bufs[key] = (torch.zeros if padded > live else torch.empty)(T, padded, dtype=adt, device=h.device)
+      return bufs[key]
+    hn = rows("hn", D, Dp)
+    x0 = None
+    if w.loop_in is not None:  # the embedding output in the operand dtype, second half of every pass's input rows
+      xx = torch.zeros(T, 2 * Dp, dtype=adt, device=h.device)
+      xx[:, Dp:Dp + D] = h.to(adt)
+    runs = self.runs
+    eps = c.rms_norm_eps
+    fresh = True  # hn does not hold this run's normed input yet
+    for j, (li, t) in enumerate(runs):
+      lw = w.layers[li]
+      s = lw.spec
+      if t >= 0:
+        xx[:, :D] = h.to(adt)
+        h = self._proj(xx, w.loop_in)[:, :D] + w.loop_step[t]
+        fresh = True
+      if fresh:
+        K.sandwich_add_norm(h, None, None, lw.norm1, eps, hn)
+      P = self._proj(hn, lw.in_w)
+      mix = rows("mix", lw.mix_cols["mix"][1], lw.out_w.shape[1])
+      self._latent_attn(P, lw, j, inp, mix, rows)
+      y = self._proj(mix, lw.out_w)
+      f = s.ffn
+      # the norm that follows this run: the next run's input norm unless a pass starts there
+      nxt = w.layers[runs[j + 1][0]].norm1 if j + 1 < len(runs) and runs[j + 1][1] < 0 else None
+      if f is None:
+        K.sandwich_add_norm(h, y, lw.norm1b, nxt, eps, hn)
+      else:
+        K.sandwich_add_norm(h, y, lw.norm1b, lw.norm2, eps, hn)
+        P = self._proj(hn, lw.ff_w)
+        if f.kind == "clamped_glu":
+          act = rows("act", f.ff, lw.down_w.shape[1])
+          K.glu_act(P, lw.ff_cols["gate"][0], lw.ff_cols["up"][0], f.ff, True, f.limit, act)
+          y = self._proj(act, lw.down_w)
+        else:
+          y = self._silu_moe(hn, P, lw, rows)
+        K.sandwich_add_norm(h, y, lw.norm2b, nxt, eps, hn)
+      fresh = nxt is None
+    if not self.shard.is_last_layer():
+      return h
+    hl = h.index_select(0, inp.last_idx)
+    xn = torch.zeros(hl.shape[0], Dp, dtype=adt, device=h.device)
+    K.sandwich_add_norm(hl, None, None, w.norm, eps, xn)
+    logits = self._proj(xn, w.lm_head)[:, :c.vocab_size]
+    if c.logit_softcap > 0:
+      logits = torch.tanh(logits / c.logit_softcap) * c.logit_softcap
+    return logits
 
   # ------------------------------------------------------------------ forward
   @torch.inference_mode()

@@ -77,6 +77,10 @@ class ShardWeights:
   norm: Optional[torch.Tensor] = None  # last shard
   lm_head: Optional[torch.Tensor] = None  # last shard (aliases embed when tied)
   vision: Optional[Dict[str, torch.Tensor]] = None  # LLaVA tower + projector (first shard), HF names
+  # looped layers (config.loop): the pass input mix [Dn, 2 D padded] over [x | embedding output] and the vector added
+  # at the start of each pass [times, D] fp32
+  loop_in: Optional[torch.Tensor] = None
+  loop_step: Optional[torch.Tensor] = None
 
   def nbytes(self) -> int:
     seen, total = set(), 0
@@ -89,7 +93,7 @@ class ShardWeights:
   def all_tensors(self) -> Iterable[torch.Tensor]:
     for lw in self.layers.values():
       yield from lw.tensors().values()
-    for t in (self.embed, self.norm, self.lm_head):
+    for t in (self.embed, self.norm, self.lm_head, self.loop_in, self.loop_step):
       if t is not None:
         yield t
     if self.vision:
@@ -339,9 +343,12 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
     for lw in sw.layers.values():
       if lw.in_w.dtype == torch.bfloat16:
         lw.in_w, lw.out_w, lw.down_w, lw.ff_w = wide(lw.in_w), wide(lw.out_w), wide(lw.down_w), wide(lw.ff_w)
+        lw.uq_w = wide(lw.uq_w)
         lw.ex_up_w, lw.ex_down_w = conv(lw.ex_up_w), conv(lw.ex_down_w)  # experts: shuffled per expert
     if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
       sw.lm_head = wide(sw.lm_head)
+    if sw.loop_in is not None and sw.loop_in.dtype == torch.bfloat16:
+      sw.loop_in = wide(sw.loop_in)
     return sw
 
   proj = conv8 if fp8 else conv
@@ -714,8 +721,17 @@ class MixedLayerWeights:
   ff_cols: Optional[Dict[str, tuple]] = None
   act: Optional[torch.Tensor] = None  # [4] fp32 PolyNorm coefficients
   router_b: Optional[torch.Tensor] = None  # [E] fp32
-  ex_up_w: Optional[torch.Tensor] = None  # [E, Fp, Dp] experts' up projections
+  ex_up_w: Optional[torch.Tensor] = None  # [E, Fp, Dp] experts' up projections ([E, 2 Fp, Dp]: gate rows, then up rows)
   ex_down_w: Optional[torch.Tensor] = None  # [E, Dq, Fp]
+  # sandwich blocks (config.block "sandwich"): norm1 / norm2 weigh the sublayers' inputs, norm1b / norm2b their
+  # results; latent attention: `in_w` = [q (or the query latent) | kv latent | rotated key part | output gate]
+  norm1b: Optional[torch.Tensor] = None  # [D] fp32
+  norm2b: Optional[torch.Tensor] = None
+  kv_norm: Optional[torch.Tensor] = None  # [kv_rank] fp32
+  q_norm: Optional[torch.Tensor] = None  # [q_rank] fp32
+  uq_w: Optional[torch.Tensor] = None  # [H (dim + rot_dim) padded, q_rank padded]
+  uk_w: Optional[torch.Tensor] = None  # [H, dim, kv_rank]: q_lat = q_unrotated . W_uk per head
+  uv_w: Optional[torch.Tensor] = None  # [H, kv_rank, vdim]: o = o_lat . W_uv^T per head (stored transposed)
 
   def tensors(self) -> Dict[str, torch.Tensor]:
     return {k: v for k, v in self.__dict__.items() if isinstance(v, torch.Tensor)}
@@ -851,6 +867,90 @@ def build_postln_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWe
   return lw
 
 
+def build_sandwich_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWeights:
+  """One sandwich layer (latent attention; clamped gated or SiLU-expert feed-forward) from `get(name)`."""
+  def dev(t, dt=torch.float32):
+    return t.to(device=device, dtype=dt).contiguous()
+  m = p + "mix."
+  a, f = spec.lattn, spec.ffn
+  blocks = [("q", get(m + "dq" if a.q_rank else m + "q")), ("ckv", get(m + "dkv"))]
+  if a.gate != "none":
+    blocks.append(("gate", get(m + "g")))
+  in_w, cols = _fused_rows(blocks, D)
+  out = get(m + "o")
+  lw = MixedLayerWeights(spec, dev(in_w, dtype), cols, dev(_pad2(out, _up(D, 64), _up(out.shape[1], 128)), dtype),
+                         {"mix": (0, out.shape[1])})
+  lw.norm1, lw.norm1b, lw.kv_norm = dev(get(p + "norm1")), dev(get(p + "norm1b")), dev(get(m + "dkv.norm"))
+  if a.q_rank:
+    lw.q_norm = dev(get(m + "dq.norm"))
+    uq = get(m + "uq")
+    lw.uq_w = dev(_pad2(uq, _up(uq.shape[0], 64), _up(a.q_rank, 128)), dtype)
+  lw.uk_w = dev(get(m + "uk").reshape(a.heads, a.dim, a.kv_rank), dtype)
+  lw.uv_w = dev(get(m + "uv").reshape(a.heads, a.vdim, a.kv_rank).transpose(1, 2), dtype)
+  if a.sink:
+    lw.sink = dev(get(m + "sink"))
+  if f is None:
+    return lw
+  q = p + "mlp."
+  if f.kind == "clamped_glu":
+    fb = [("gate", get(q + "gate")), ("up", get(q + "up"))]
+    down = get(q + "down")
+  else:
+    fb = [("router", get(q + "router"))]
+    down = None
+    if f.shared_ff:
+      fb += [("sh_gate", get(q + "shared.gate")), ("sh_up", get(q + "shared.up"))]
+      down = get(q + "shared.down")
+    Fp, Dp = _up(f.ff, 128), _up(D, 128)
+    lw.ex_up_w = dev(torch.stack([torch.cat([_pad2(get(q + f"e{e}.gate"), Fp, Dp), _pad2(get(q + f"e{e}.up"), Fp, Dp)])
+                                  for e in range(f.experts)]), dtype)
+    lw.ex_down_w = dev(torch.stack([_pad2(get(q + f"e{e}.down"), Dp, Fp) for e in range(f.experts)]), dtype)
+  ff_w, lw.ff_cols = _fused_rows(fb, D)
+  lw.ff_w = dev(ff_w, dtype)
+  if down is not None:
+    lw.down_w = dev(_pad2(down, _up(D, 64), _up(down.shape[1], 128)), dtype)
+  lw.norm2, lw.norm2b = dev(get(p + "norm2")), dev(get(p + "norm2b"))
+  return lw
+
+
+def sandwich_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
+  """Name -> shape of every tensor of a sandwich-block checkpoint (Nenizen); the LM head is the embedding table."""
+  D, out = c.hidden_size, {}
+  out["embed"] = (c.vocab_size, D)
+  if c.loop:
+    out["loop.in"], out["loop.step"] = (D, 2 * D), (c.loop[2], D)
+  for i, s in enumerate(c.layer_specs):
+    p, m, a, f = f"l{i}.", f"l{i}.mix.", s.lattn, s.ffn
+    out[p + "norm1"], out[p + "norm1b"] = (D,), (D,)
+    qd = a.heads * (a.dim + a.rot_dim)
+    if a.q_rank:
+      out[m + "dq"], out[m + "dq.norm"], out[m + "uq"] = (a.q_rank, D), (a.q_rank,), (qd, a.q_rank)
+    else:
+      out[m + "q"] = (qd, D)
+    out[m + "dkv"], out[m + "dkv.norm"] = (a.kv_rank + a.rot_dim, D), (a.kv_rank,)
+    out[m + "uk"], out[m + "uv"] = (a.heads * a.dim, a.kv_rank), (a.heads * a.vdim, a.kv_rank)
+    if a.gate != "none":
+      out[m + "g"] = (a.gate_rows, D)
+    if a.sink:
+      out[m + "sink"] = (a.heads,)
+    out[m + "o"] = (D, a.heads * a.vdim)
+    if f is None:
+      continue
+    q = p + "mlp."
+    out[p + "norm2"], out[p + "norm2b"] = (D,), (D,)
+    if f.kind == "clamped_glu":
+      out[q + "gate"], out[q + "up"], out[q + "down"] = (f.ff, D), (f.ff, D), (D, f.ff)
+    else:
+      for e in range(f.experts):
+        out[q + f"e{e}.gate"], out[q + f"e{e}.up"], out[q + f"e{e}.down"] = (f.ff, D), (f.ff, D), (D, f.ff)
+      out[q + "router"] = (f.experts, D)
+      if f.shared_ff:
+        out[q + "shared.gate"], out[q + "shared.up"], out[q + "shared.down"] = (f.shared_ff, D), (f.shared_ff, D), \
+          (D, f.shared_ff)
+  out["final.norm"] = (D,)
+  return out
+
+
 def postln_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
   """Name -> shape of every tensor of a post-norm mixed-layer checkpoint (Mogelix)."""
   D, out = c.hidden_size, {}
@@ -893,6 +993,8 @@ def mixed_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
   """Name -> shape of every tensor of a mixed-layer checkpoint (random init, checkpoint validation)."""
   if c.block == "postln":
     return postln_tensor_shapes(c)
+  if c.block == "sandwich":
+    return sandwich_tensor_shapes(c)
   D, out = c.hidden_size, {}
   out["embed"] = (c.vocab_size, D)
   for i, s in enumerate(c.layer_specs):
@@ -931,7 +1033,7 @@ def random_mixed_tensors(c: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
       t = torch.randn(shape, generator=g) * 0.5
     elif leaf in ("sink", "D", "act") or (leaf == "b" and c.block == "postln"):
       t = torch.randn(shape, generator=g) * (0.5 if leaf == "b" else 1.0)
-    elif leaf in ("norm1", "norm2") or name == "final.norm":
+    elif leaf in ("norm1", "norm2", "norm1b", "norm2b") or name == "final.norm":
       t = 1.0 + 0.1 * torch.randn(shape, generator=g)
     elif leaf in ("ls1", "ls2"):
       t = 0.5 + 0.1 * torch.randn(shape, generator=g)
@@ -943,8 +1045,10 @@ def random_mixed_tensors(c: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
       t = torch.rand(shape, generator=g) * 1.5 - 2.0
     elif leaf == "b" and len(shape) == 1:  # a2.b: decays close to one
       t = 3.0 + torch.randn(shape, generator=g)
+    elif name == "loop.step":
+      t = torch.randn(shape, generator=g) * 0.3
     elif name == "embed":
-      t = torch.randn(shape, generator=g)
+      t = torch.randn(shape, generator=g) * (0.25 if c.block == "sandwich" else 1.0)
     else:
       t = torch.randn(shape, generator=g) / shape[-1] ** 0.5
     out[name] = t.to(torch.bfloat16).float()
@@ -955,15 +1059,23 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
   """ShardWeights of a mixed-layer model from `get(name) -> fp32 CPU tensor`."""
   sw = ShardWeights(c, shard)
   D = c.hidden_size
-  build = build_postln_layer if c.block == "postln" else build_mixed_layer
+  build = {"postln": build_postln_layer, "sandwich": build_sandwich_layer}.get(c.block, build_mixed_layer)
   for i in shard.layers():
     sw.layers[i] = build(c.layer_specs[i], get, f"l{i}.", D, device, dtype)
   if shard.is_first_layer():
-    sw.embed = get("embed").to(device=device, dtype=torch.float32).contiguous()  # gathered into the fp32 residual
+    # gathered into the fp32 residual; a model that scales its embedding output gathers from the scaled table
+    sw.embed = (get("embed") * c.embed_scale).to(device=device, dtype=torch.float32).contiguous()
+  if c.loop and any(c.loop[0] <= i < c.loop[1] for i in shard.layers()):
+    w_in = get("loop.in")  # [D, 2 D] over [x | embedding output]: each half padded to the GEMM's K tile
+    Dp = _up(D, 128)
+    li = torch.zeros(_up(D, 64), 2 * Dp)
+    li[:D, :D], li[:D, Dp:Dp + D] = w_in[:, :D], w_in[:, D:]
+    sw.loop_in = li.to(device=device, dtype=dtype).contiguous()
+    sw.loop_step = get("loop.step").to(device=device, dtype=torch.float32).contiguous()
   if shard.is_last_layer():
     sw.norm = get("final.norm").reshape(-1).to(device=device, dtype=torch.float32)
     head = torch.zeros(_up(c.vocab_size, 64), _up(D, 128))
-    head[:c.vocab_size, :D] = get("head")
+    head[:c.vocab_size, :D] = get("embed" if c.tie_word_embeddings and c.is_mixed else "head")
     sw.lm_head = head.to(device=device, dtype=dtype).contiguous()
   return sw
 
@@ -984,8 +1096,10 @@ def load_mixed_weights(model_dir: Path, c: ModelConfig, shard: Shard, device, dt
     return handles[f].get_tensor(name).float()
   want = mixed_tensor_shapes(c)
   for name, shape in want.items():
-    if name.split(".")[0] in ("embed", "final", "head") or int(name.split(".")[0][1:]) in shard.layers():
+    if name.split(".")[0] in ("embed", "final", "head", "loop") or int(name.split(".")[0][1:]) in shard.layers():
       got = tuple(get(name).shape) if not name.endswith((".a1", ".a2")) else None
+      if name == "loop.step" and got is not None and got[1:] == tuple(shape)[1:] and got[0] >= shape[0]:
+        continue
       if got is not None and got != tuple(shape):
         raise ValueError(f"{name}: checkpoint shape {got}, config says {tuple(shape)}")
   return mixed_weights(c, shard, get, device, dtype)

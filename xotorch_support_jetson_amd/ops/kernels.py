@@ -561,3 +561,50 @@ def moe_weighted_sum(y, slot_of, topw, k: int, sh_y, P, shg_off: int, out, split
   """out [T, D] fp32 = sum_j topw[t, j] * y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) * sh_y[t] for a shared expert);
   y [splits * T k, >= D]: the experts' down projections, K slice after K slice."""
   _mix("moe_weighted_sum", _gpu(y))(y, slot_of, topw, int(k), sh_y, P, int(shg_off), out, int(splits))
+
+
+# ------------------------------------------------------------------ sandwich blocks (csrc/latent.hip)
+def sandwich_add_norm(x, y, wb, wn, eps: float, out=None) -> None:
+  """fp32 stream rows x [T, D] += y / rms(y) * wb in place (y None: nothing is added); with wn, out[:, :D] =
+  x / rms(x) * wn in out's dtype (the next GEMM's operand)."""
+  _mix("sandwich_add_norm", _gpu(x))(x, y, wb, wn, float(eps), out)
+
+
+def latent_kv_store(P, ckv_off: int, R: int, dr: int, kv_norm, q_off: int, q_rank: int, q_norm, eps: float, rot_dims: int,
+                    interleaved: bool, pos, cos_sin, slots, cache, qa_out) -> None:
+  """Per token: the latent rms_norm(P[:, ckv_off : +R]) * kv_norm and the rotated key part rope(P[:, ckv_off + R : +dr])
+  -> cache [pages, 1, 64, R + dr] at `slots`; q_rank > 0: qa_out[:, :q_rank] = rms_norm(P[:, q_off : +q_rank]) * q_norm
+  (the query latent, operand of the query up-projection).  RoPE on the first rot_dims dims of the rotated part, pairs
+  (2i, 2i + 1) (interleaved) or (i, i + rot_dims / 2); cos_sin [rows, rot_dims] = (cos | sin)."""
+  _mix("latent_kv_store", _gpu(P))(P, int(ckv_off), int(R), int(dr), kv_norm, int(q_off), int(q_rank), q_norm, float(eps),
+                                   int(rot_dims), bool(interleaved), pos, cos_sin, slots, cache, qa_out)
+
+
+def latent_q_rope(Q, q_off: int, H: int, dn: int, dr: int, rot_dims: int, interleaved: bool, pos, cos_sin, qn_out,
+                  qpe_out) -> None:
+  """Queries Q[:, q_off : +H (dn + dr)], head by head [dn unrotated | dr rotated]: the unrotated parts -> qn_out
+  [H, T, dn] (operand of the per-head product with W_uk), the rotated parts after RoPE -> qpe_out [T, H, dr]."""
+  _mix("latent_q_rope", _gpu(Q))(Q, int(q_off), int(H), int(dn), int(dr), int(rot_dims), bool(interleaved), pos, cos_sin,
+                                 qn_out, qpe_out)
+
+
+def latent_attn(q_lat, q_pe, cache, block_tables, cu_q, ctx_lens, sink, scale: float, window: int, out,
+                max_qlen: int = 0) -> None:
+  """out [H, T, R] = softmax attention of every head's absorbed query (q_lat [H, T, R] against the cached latents, q_pe
+  [T, H, dr] against the cached rotated key parts, times scale) over the tokens at most window - 1 places back
+  (window 0: all earlier ones), the values being the latents themselves; sink [H] (or None): one more logit per head in
+  the denominator.  cache [pages, 1, 64, R + dr]."""
+  _mix("latent_attn", _gpu(q_lat))(q_lat, q_pe, cache, block_tables, cu_q, ctx_lens, sink, float(scale), int(window), out,
+                                   int(max_qlen) or int(q_lat.shape[1]))
+
+
+def latent_out_gate(o, P, g_off: int, gate: int, out) -> None:
+  """o [H, T, dv] -> out[:, :H dv] (token-major, out's dtype) times sigmoid(P[:, g_off : ...]): gate 0 none, 1 one
+  gate per element, 2 one per head."""
+  _mix("latent_out_gate", _gpu(o))(o, P, int(g_off), int(gate), out)
+
+
+def glu_act(P, gate_off: int, up_off: int, F: int, clamped: bool, limit: float, out) -> None:
+  """out[:, :F] = silu(g) * u, or (clamped) g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u,
+  -limit, limit); g = P[:, gate_off : +F], u = P[:, up_off : +F]."""
+  _mix("glu_act", _gpu(P))(P, int(gate_off), int(up_off), int(F), bool(clamped), float(limit), out)

@@ -498,5 +498,100 @@ def moe_weighted_sum(y, slot_of, topw, k, sh_y, P, shg_off, out, splits=1):
   y = y.reshape(splits, T * k, -1).float().sum(0)
   acc = (y[slot_of.long().reshape(T, k), :D] * topw.reshape(T, k, 1)).sum(1)
   if sh_y is not None:
-    acc = acc + torch.sigmoid(P[:, shg_off:shg_off + 1].float()) * sh_y[:, :D].float()
+    sh = sh_y[:, :D].float()
+    acc = acc + (sh if P is None else torch.sigmoid(P[:, shg_off:shg_off + 1].float()) * sh)
   out.copy_(acc)
+
+
+# ------------------------------------------------------------------ sandwich blocks: latent attention, gated feed-forwards
+# Torch twins of csrc/latent.hip.
+def sandwich_add_norm(x, y, wb, wn, eps, out):
+  """x += y / rms(y) * wb in place (y None: nothing is added); with wn, out[:, :D] = x / rms(x) * wn."""
+  D = x.shape[1]
+  if y is not None:
+    yy = y[:, :D].float()
+    x += yy / torch.sqrt(yy.pow(2).mean(-1, keepdim=True) + eps) * wb.float()
+  if wn is not None:
+    out[:, :D] = (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * wn.float()).to(out.dtype)
+
+
+def _rope_pairs(x, cs, R, interleaved):
+  """x [T, heads, d]: the first R dims rotated by the table rows cs [T, R] = (cos | sin); partner of dim 2i is 2i + 1
+  (interleaved) or of dim i is i + R / 2."""
+  if not R:
+    return x
+  half = R // 2
+  c, s = cs[:, None, :half], cs[:, None, half:]
+  x = x.clone()
+  if interleaved:
+    a, b = x[..., 0:R:2].clone(), x[..., 1:R:2].clone()
+    x[..., 0:R:2], x[..., 1:R:2] = a * c - b * s, b * c + a * s
+  else:
+    a, b = x[..., :half].clone(), x[..., half:R].clone()
+    x[..., :half], x[..., half:R] = a * c - b * s, b * c + a * s
+  return x
+
+
+def latent_kv_store(P, ckv_off, R, dr, kv_norm, q_off, q_rank, q_norm, eps, rot_dims, interleaved, pos, cos_sin, slots,
+                    cache, qa_out):
+  T = P.shape[0]
+  c = P[:, ckv_off:ckv_off + R].float()
+  c = c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kv_norm.float()
+  kr = P[:, ckv_off + R:ckv_off + R + dr].float().reshape(T, 1, dr)
+  kr = _rope_pairs(kr, cos_sin[pos.long()] if rot_dims else None, rot_dims, interleaved).reshape(T, dr)
+  ok = slots >= 0
+  s = slots[ok].long()
+  cache[s // PAGE, 0, s % PAGE] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+  if q_rank:
+    q = P[:, q_off:q_off + q_rank].float()
+    qa_out[:, :q_rank] = (q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.float()).to(qa_out.dtype)
+
+
+def latent_q_rope(Q, q_off, H, dn, dr, rot_dims, interleaved, pos, cos_sin, qn_out, qpe_out):
+  T = Q.shape[0]
+  q = Q[:, q_off:q_off + H * (dn + dr)].float().reshape(T, H, dn + dr)
+  qn_out.copy_(q[..., :dn].transpose(0, 1).to(qn_out.dtype))
+  qpe_out.copy_(_rope_pairs(q[..., dn:], cos_sin[pos.long()] if rot_dims else None, rot_dims, interleaved).to(qpe_out.dtype))
+
+
+def latent_attn(q_lat, q_pe, cache, block_tables, cu_q, ctx_lens, sink, scale, window, out, max_qlen=0):
+  H, T, R = q_lat.shape
+  for b in range(ctx_lens.numel()):
+    t0, t1, n = int(cu_q[b]), int(cu_q[b + 1]), int(ctx_lens[b])
+    if n <= 0 or t1 == t0:
+      continue
+    npg = -(-n // PAGE)
+    rows = cache[block_tables[b, :npg].long(), 0].reshape(npg * PAGE, -1)[:n].float()
+    qpos = torch.arange(n - (t1 - t0), n)[:, None]
+    kpos = torch.arange(n)[None, :]
+    vis = kpos <= qpos
+    if window:
+      vis = vis & (qpos - kpos < window)
+    s = (torch.einsum("htr,jr->htj", q_lat[:, t0:t1].float(), rows[:, :R]) +
+         torch.einsum("thr,jr->htj", q_pe[t0:t1].float(), rows[:, R:])) * scale
+    s = s.masked_fill(~vis[None], float("-inf"))
+    if sink is not None:
+      s = torch.cat([s, sink.float()[:, None, None].expand(H, t1 - t0, 1)], -1)
+    w = torch.softmax(s, -1)[..., :n]
+    out[:, t0:t1] = torch.einsum("htj,jr->htr", w, rows[:, :R]).to(out.dtype)
+
+
+def latent_out_gate(o, P, g_off, gate, out):
+  """o [H, T, dv] -> out[:, :H dv] token-major, times sigmoid of P's gate columns: gate 1 one per element, 2 one per head."""
+  H, T, dv = o.shape
+  y = o.float().transpose(0, 1)
+  if gate == 1:
+    y = y * torch.sigmoid(P[:, g_off:g_off + H * dv].float()).reshape(T, H, dv)
+  elif gate == 2:
+    y = y * torch.sigmoid(P[:, g_off:g_off + H].float()).reshape(T, H, 1)
+  out[:, :H * dv] = y.reshape(T, H * dv).to(out.dtype)
+
+
+def glu_act(P, gate_off, up_off, Fd, clamped, limit, out):
+  g, u = P[:, gate_off:gate_off + Fd].float(), P[:, up_off:up_off + Fd].float()
+  if clamped:
+    g, u = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+    y = g * torch.sigmoid(1.702 * g) * (u + 1)
+  else:
+    y = F.silu(g) * u
+  out[:, :Fd] = y.to(out.dtype)
