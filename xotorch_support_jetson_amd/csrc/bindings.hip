@@ -8,6 +8,7 @@
 namespace xot {
 void bind_mixers(pybind11::module& m);  // csrc/mixers.hip
 void bind_hybrid(pybind11::module& m);  // csrc/hybrid.hip
+void bind_latent(pybind11::module& m);  // csrc/latent.hip
 }
 
 namespace {
@@ -1021,6 +1022,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "xot MI355X (gfx950) kernel library";
   xot::bind_mixers(m);
   xot::bind_hybrid(m);
+  xot::bind_latent(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("rmsnorm_bwd", &rmsnorm_bwd, py::arg("x"), py::arg("w"), py::arg("dy"), py::arg("dx"), py::arg("dw"),
         py::arg("eps"), py::arg("res") = py::none());

@@ -10,7 +10,7 @@
 //   ssd_gate_norm       (o + D x) * silu(z), RMS norm in equal groups, weight
 //   polynorm_act        a N(z) + b N(z^2) + c N(z^3) + e with N = division by the row's RMS
 //   relu2               relu(z)^2
-//   moe_weighted_sum    sum_j w_j y[slot_j] + sigmoid(gate) * shared
+//   moe_weighted_sum    sum_j w_j y[slot_j] + sigmoid(gate) * shared (or + shared, ungated)
 //
 // P is a fused projection's fp32 output [T, ldp]; "column offset" arguments address its slices.  Activations that
 // feed the next GEMM (AT) are bf16 or fp32; norms, scores, softmax weights, gates and everything a recurrence reads
@@ -687,7 +687,7 @@ __global__ void moe_weighted_sum_k(const float* __restrict__ y, int ldy, const i
                                    const float* __restrict__ sh, int lds, const float* __restrict__ P, int ldp, int shg_off,
                                    float* __restrict__ out, int D) {
   const int64_t t = blockIdx.x;
-  const float sg = sh ? sigmoidf_(P[t * ldp + shg_off]) : 0.0f;
+  const float sg = !sh ? 0.0f : (P ? sigmoidf_(P[t * ldp + shg_off]) : 1.0f);  // (no gate: the shared expert is added as it is)
   for (int i = threadIdx.x; i < D; i += blockDim.x) {
     float acc = 0.0f;
     for (int j = 0; j < k; ++j) {
@@ -1037,12 +1037,14 @@ void moe_weighted_sum(const at::Tensor& y, const at::Tensor& slot_of, const at::
   int lds = 0, ldp = 0;
   if (sh_y.has_value()) {
     lds = ld_of(*sh_y, "sh_y");
-    MCHECK(P.has_value() && sh_y->size(0) == T && sh_y->size(1) >= D, "a shared expert needs its result [T, >= D] and its gate");
-    ldp = ld_of(*P, "P");
-    MCHECK(P->size(0) == T, "P must have T rows");
-    cols_ok(*P, shg_off, 1, "shared gate");
+    MCHECK(sh_y->size(0) == T && sh_y->size(1) >= D, "a shared expert needs its result [T, >= D]");
     sp = sh_y->data_ptr<float>();
-    pp = P->data_ptr<float>();
+    if (P.has_value()) {
+      ldp = ld_of(*P, "P");
+      MCHECK(P->size(0) == T, "P must have T rows");
+      cols_ok(*P, shg_off, 1, "shared gate");
+      pp = P->data_ptr<float>();
+    }
   }
   // (slot_of comes from the routing kernel: every entry is a row of y)
   moe_weighted_sum_k<<<T, 256, 0, stream()>>>(y.data_ptr<float>(), ldy, slot_of.data_ptr<int>(), topw.data_ptr<float>(), (int)k,

@@ -1081,7 +1081,7 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
 
 
 def load_mixed_weights(model_dir: Path, c: ModelConfig, shard: Shard, device, dtype) -> ShardWeights:
-  """Tarepel / Mogelix checkpoint (flat names: embed, l<i>.norm1, l<i>.mix.*, l<i>.mlp.*, l<i>.ls1 / ls2 or l<i>.rg1 /
+  """Tarepel / Mogelix / Nenizen checkpoint (flat names: embed, l<i>.norm1, l<i>.mix.*, l<i>.mlp.*, l<i>.ls1 / ls2 or l<i>.rg1 /
   rg2, final.norm, head).  The decay rank of a gated-linear-attention layer is the a1 tensor's row count."""
   from safetensors import safe_open
   wm = _weight_map(Path(model_dir))
