@@ -167,7 +167,11 @@ __global__ __launch_bounds__(64 * LATT_WAVES) void latent_attn_k(
   const int t = blockIdx.x, h0 = blockIdx.y * REP;
   const int b = seq_of(cu_q, B, t);
   const int ctx = ctx_lens[b];
-  if (ctx <= 0) return;  // padding row of a captured decode batch
+  if (ctx <= 0) {  // padding row of a captured decode batch: zeros, so that nothing downstream reads stale memory
+    for (int e = threadIdx.x; e < REP * R; e += blockDim.x)
+      if (h0 + e / R < H) stf(out + ((int64_t)(h0 + e / R) * T + t) * R + e % R, 0.0f);
+    return;
+  }
   const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
   for (int i = threadIdx.x; i < REP * d; i += blockDim.x) {
     const int r = i / d, e = i - r * d, h = min(h0 + r, H - 1);

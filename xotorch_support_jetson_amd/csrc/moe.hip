@@ -195,6 +195,9 @@ __global__ __launch_bounds__(256) void moe_topk_ds_kernel(const float* __restric
         id = oi;
       }
     }
+    // (scores that are not numbers -- rows of a padded batch may hold anything -- leave no winner: take expert j,
+    // so that every index written below is an expert)
+    if (id >= E) id = j;
     // the owner lane retires the winner and contributes its score
     float wv = 0.f;
 #pragma unroll
