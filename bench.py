@@ -155,6 +155,36 @@ def hybrid_configs(name: str):
   return hybrid, mixer_configs(name)[0]
 
 
+def latent_configs(name: str):
+  """(Nenizen-design config, the closest existing model: a DeepSeek-V2-style stack with the same latent attention
+  sizes -- latent 256, 64 rotated and 128 unrotated key dims, 128 value dims per head -- width, depth, heads and
+  experts).  Nenizen layers in turn: causal with an element-wise output gate under a clamped gated feed-forward; causal
+  with a sink under 8 SiLU experts, 2 chosen, plus a shared expert; sliding window (the size's chunk) with a per-head
+  gate under the dense feed-forward; the sink layer again.  No loop (equal depth on both sides)."""
+  from xotorch_support_jetson_amd.models.config import ModelConfig, from_hf_config
+  z = MIXER_SIZES[name]
+  H, _, _, chunk, _ = z["attn"]
+  W, qr = z["width"], z["width"] // 2
+  fe = (z["ff"] // 2 + 127) // 128 * 128
+  mix = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 256, "scale": 192 ** -0.5}
+  dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+  moe = {"kind": "moe", "expert": {"ff": fe}, "router": {"experts": 8, "top": 2}, "shared": {"ff": fe}}
+  kinds = [
+    {"type": "latent_attention", "mlp": dense, "mixer": dict(mix, rot={"base": 1e6, "dims": 64})},
+    {"type": "latent_attention_3", "mlp": moe, "mixer": dict(mix, q_rank=qr, rot={"base": 1e4, "dims": 64})},
+    {"type": "latent_attention_2", "mlp": dense,
+     "mixer": dict(mix, q_rank=qr, rot={"base": 1e6, "dims": 64}, mask={"size": chunk})},
+  ]
+  latent = from_hf_config({"architecture": "Nenizen", "vocab": 32000, "width": W, "norm": {"eps": 1e-5},
+                           "embedding": {"scale": 1.0}, "logit_softcap": 30.0,
+                           "layers": [kinds[(0, 1, 2, 1)[i % 4]] for i in range(z["layers"])]})
+  ds = ModelConfig("deepseek_v2", 32000, W, z["ff"], z["layers"], H, 1, 192, 1e-5, 1e4, None, 32768, False,
+                   num_experts=8, num_experts_per_tok=2, bos_token_id=1, eos_token_ids=(2,), q_lora_rank=qr,
+                   kv_lora_rank=256, qk_nope_head_dim=128, qk_rope_head_dim=64, v_head_dim=128, moe_intermediate_size=fe,
+                   n_shared_experts=1, first_k_dense_replace=0, moe_layer_freq=2, norm_topk_prob=False)
+  return latent, ds
+
+
 def bench_mixers(args, sizes=None, kinds=("tarepel", "llama"), configs=mixer_configs,
                  what="Tarepel-design layers beside a Llama-style stack of equal size"):
   """Prefill and decode throughput of mixed-layer designs at sizes like a real model's (random weights), beside
@@ -232,7 +262,11 @@ def main():
   ap.add_argument("--hybrid", default=None, metavar="SIZES",
                   help="instead of the headline: Mogelix-design layers (window attention with pooled blocks, Mamba-2, "
                        "relu^2 experts) beside the Tarepel-design stack at the named sizes; one GPU")
-  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers / --hybrid: sequences per step")
+  ap.add_argument("--latent", default=None, metavar="SIZES",
+                  help="instead of the headline: Nenizen-design layers (latent attention with window / sink / output "
+                       "gates, clamped gated feed-forward, SiLU experts) beside a DeepSeek-V2-style stack of the same "
+                       "latent sizes at the named sizes; one GPU")
+  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers / --hybrid / --latent: sequences per step")
   args = ap.parse_args()
   os.environ["XOT_WEIGHT_DTYPE"] = args.weight_dtype
   if args.mixers:
@@ -240,6 +274,10 @@ def main():
   if args.hybrid:
     return bench_mixers(args, args.hybrid, ("mogelix", "tarepel"), hybrid_configs,
                         "Mogelix-design layers beside a Tarepel-design stack of equal size")
+
+  if args.latent:
+    return bench_mixers(args, args.latent, ("nenizen", "deepseek"), latent_configs,
+                        "Nenizen-design layers beside a DeepSeek-V2-style stack of equal size")
 
   from xotorch_support_jetson_amd.models.config import preset
   from xotorch_support_jetson_amd.parallel.comm import P2PTransport, init_distributed

@@ -130,7 +130,7 @@ class Rig:
       if max(L["mlp"]["router"]["experts"] for L in self.cfg["layers"] if L.get("mlp") and L["mlp"]["kind"] == "moe") > 16:
         # dozens of experts with near-uniform scores: the chosen sets differ at many positions in bf16 (the torch twins
         # in bf16 show the same); only the typical position is checked, the float32 runs pin the mechanism
-        assert err.median() < TOL[self.dtype] / 2, f"{what}: median error {float(err.median()):.3g}"
+        assert err.median() < TOL[self.dtype], f"{what}: median error {float(err.median()):.3g}"
         return
       assert over <= max(2, len(toks) // 12) and err.median() < TOL[self.dtype] / 3, \
         f"{what}: {over} of {len(toks)} positions off, the worst ({worst}) by {float(err.max()):.3g}"
