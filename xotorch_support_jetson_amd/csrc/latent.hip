@@ -17,6 +17,13 @@ namespace xot {
 namespace {
 using namespace mix;
 
+typedef __attribute__((address_space(3))) s16x4* lds_s16x4_t;
+// transposed LDS read (gfx950): within each group of 16 lanes, lane 4 q + p gives the address of 4 consecutive 16-bit
+// elements (row q, columns 4 p .. 4 p + 3 of a 4 x 16 block); lane c receives column c of rows 0 .. 3
+__device__ __forceinline__ s16x4 tr_read(const uint16_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t)(p));
+}
+
 constexpr float LOG2E_F = 1.4426950408889634f;
 
 // ------------------------------------------------------------------ residual add of a normed sublayer result + next norm
@@ -281,77 +288,124 @@ __global__ __launch_bounds__(64 * LATT_WAVES) void latent_attn_k(
   }
 }
 
-// ------------------------------------------------------------------ MFMA kernel for prompt portions (bf16)
-// A workgroup owns 64 consecutive new tokens of one (sequence, head), 16 per wave, and walks the pages from its first
-// query's window (or the sequence's start) to its last query: a page's 64 rows are staged in LDS row-major (the K
-// operand; row length padded with zeros to a multiple of 32) and, their latent part, transposed (the V^T operand).
-// Scores are computed transposed, S^T = K Q^T (keys x queries, 16x16x32 MFMA), so a lane's accumulator rows are keys of
-// ONE query: running maximum and denominator are per lane (the four lanes of a query agree on the maximum through two
-// shuffles and keep partial denominators), and the exponentials, rounded to bf16, are as they lie the B operand of
-// O^T += V^T P^T, whose k slots (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.  Scores,
-// maxima and sums are fp32 (base-2 exponentials of scores scaled by log2 e); a sink's logit starts the running
-// maximum with a denominator of one.  NV: compile-time bound on R / 16 (the output accumulators).
+// ------------------------------------------------------------------ MFMA kernel (bf16): prompt portions and single tokens
+// Columns of a wave's 16x16 tiles are 16 (query, head) pairs that share the keys: in a prompt portion (DEC false) a
+// workgroup of four waves owns 64 consecutive new tokens of one (sequence, head), 16 per wave; for single tokens (DEC
+// true) a one-wave workgroup owns one token's block of 16 heads and one share of its pages (key split), and writes
+// (maximum, denominator, sums) partials that latent_attn_merge_k adds up.  A page's 64 rows are staged in LDS row-major
+// (row length padded with zeros to a multiple of 32); the queries sit in registers as B operands.
+// Scores are computed transposed, S^T = K Q^T (keys x columns, 16x16x32 MFMA), so a lane's accumulator rows are keys
+// of ONE column: running maximum and denominator are per lane (the four lanes of a column agree on the maximum through
+// two shuffles and keep partial denominators), and the exponentials, rounded to bf16, are as they lie the B operand of
+// O^T += V^T P^T, whose k slots (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.  The V^T
+// operand comes straight out of the row-major page image by the transposed LDS read (4 keys x 16 dims per 16 lanes).
+// Scores, maxima and sums are fp32 (base-2 exponentials of scores scaled by log2 e); a sink's logit starts the
+// running maximum with a denominator of one.  NV: compile-time bound on R / 16 (output accumulators); the row length
+// is at most 32 (NV / 2 + 2).
 constexpr int LM_PAD = 8;
 
-template <int NV>
-__global__ __launch_bounds__(256) void latent_attn_mfma_k(
+template <int NV, bool DEC>
+__global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
     const uint16_t* __restrict__ q_lat, const uint16_t* __restrict__ q_pe, const uint16_t* __restrict__ cache,
-    const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int T,
-    const float* __restrict__ sink, float scale_l2, int window, uint16_t* __restrict__ out, int H, int R, int dr) {
+    const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int B,
+    int T, const float* __restrict__ sink, float scale_l2, int window, uint16_t* __restrict__ out, float* __restrict__ part,
+    int nsplit, int H, int R, int dr) {
+  constexpr int NQ = NV / 2 + 2, NT = DEC ? 64 : 256, QROWS = DEC ? 16 : 64;
   extern __shared__ __attribute__((aligned(16))) uint16_t lsm[];
-  const int b = blockIdx.y, h = blockIdx.z, q0 = blockIdx.x * 64;
-  const int n = ctx_lens[b], t0 = cu_q[b], ql = cu_q[b + 1] - t0;
-  if (n <= 0 || q0 >= ql) return;
-  const int base = n - ql;
-  const int DK = R + dr, DKp = (DK + 31) & ~31, LDK = DKp + LM_PAD, LDV = PAGE_TOK + LM_PAD;
-  const int nv = R >> 4;
-  uint16_t* Qs = lsm;                 // [64][LDK]
-  uint16_t* Ks = Qs + 64 * LDK;       // [64][LDK]
-  uint16_t* Vt = Ks + 64 * LDK;       // [R][LDV]
+  const int DK = R + dr, DKp = (DK + 31) & ~31, LDK = DKp + LM_PAD;
+  const int nv = R >> 4, nq = DKp >> 5;
+  uint16_t* Qs = lsm;                 // [QROWS][LDK]
+  uint16_t* Ks = Qs + QROWS * LDK;    // [64][LDK]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, lq = lane & 15;
+  int b, h0 = 0, t0 = 0, ql = 0, q0 = 0, base = 0, tok = 0;
+  if constexpr (DEC) {
+    tok = blockIdx.z;
+    h0 = blockIdx.y * 16;
+    b = seq_of(cu_q, B, tok);
+  } else {
+    b = blockIdx.y;
+    h0 = blockIdx.z;
+    q0 = blockIdx.x * 64;
+  }
+  const int n = ctx_lens[b];
+  t0 = cu_q[b];
+  ql = cu_q[b + 1] - t0;
+  base = n - ql;
+  const int head = DEC ? min(h0 + lq, H - 1) : h0;
+  if constexpr (DEC) {
+    if (n <= 0) {  // padding row of a captured decode batch: zeros, an empty partial
+      if (h0 + lq < H) {
+        if (nsplit == 1) {
+          for (int i = g; i < R; i += 4) out[((int64_t)head * T + tok) * R + i] = 0;
+        } else {
+          float* pr = part + (((int64_t)tok * H + head) * nsplit + blockIdx.x) * (2 + R);
+          for (int i = g; i < 2 + R; i += 4) pr[i] = i == 0 ? -INFINITY : 0.0f;
+        }
+      }
+      return;
+    }
+  } else {
+    if (n <= 0 || q0 >= ql) return;
+  }
   const int* bt = block_tables + (int64_t)b * width;
-  // queries -> LDS (rows past the sequence's new tokens and the padding columns: zero)
+  // queries -> LDS (rows without a query and the padding columns: zero), then into registers as B operands
   const int chunks = DKp >> 3;
-  for (int idx = tid; idx < 64 * chunks; idx += 256) {
+  for (int idx = tid; idx < QROWS * chunks; idx += NT) {
     const int row = idx / chunks, dim = (idx - row * chunks) << 3;
     s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (q0 + row < ql && dim < DK) {
-      const int64_t t = t0 + q0 + row;
-      v = dim < R ? ld16(q_lat + ((int64_t)h * T + t) * R + dim) : ld16(q_pe + (t * H + h) * dr + (dim - R));
+    const bool has = DEC ? (h0 + row < H) : (q0 + row < ql);
+    if (has && dim < DK) {
+      const int64_t t = DEC ? tok : t0 + q0 + row;
+      const int hh = DEC ? h0 + row : h0;
+      v = dim < R ? ld16(q_lat + ((int64_t)hh * T + t) * R + dim) : ld16(q_pe + (t * H + hh) * dr + (dim - R));
     }
     st16(Qs + row * LDK + dim, v);
-    if (dim >= DK) st16(Ks + row * LDK + dim, v);  // the keys' padding columns stay zero
   }
-  const int qi = q0 + 16 * wave + lq;      // this lane's query (new-token index in the sequence)
-  const bool valid = qi < ql;
-  const int qp = base + qi;                // its position
-  const int wq_lo = base + q0 + 16 * wave, wq_hi = base + min(q0 + 16 * wave + 15, ql - 1);  // the wave's positions
+  for (int idx = tid; idx < 64 * ((DKp - DK) >> 3); idx += NT) {  // the keys' padding columns stay zero
+    const int pc = (DKp - DK) >> 3, row = idx / pc, dim = DK + ((idx - row * pc) << 3);
+    st16(Ks + row * LDK + dim, s16x8{0, 0, 0, 0, 0, 0, 0, 0});
+  }
+  __syncthreads();
+  s16x8 qreg[NQ];
+  {
+    const uint16_t* qb = Qs + ((DEC ? 0 : 16 * wave) + lq) * LDK + 8 * g;
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) qreg[i] = i < nq ? ld16(qb + 32 * i) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  // this lane's column: its query's position, whether it is a real one
+  const int qi = DEC ? 0 : q0 + 16 * wave + lq;
+  const bool valid = DEC ? (h0 + lq < H) : (qi < ql);
+  const int qp = DEC ? base + (tok - t0) : base + qi;
+  const int wq_lo = DEC ? qp : base + q0 + 16 * wave;                       // the wave's positions
+  const int wq_hi = DEC ? qp : base + min(q0 + 16 * wave + 15, ql - 1);
+  const int first = DEC ? (window > 0 ? max(0, qp - window + 1) : 0) : (window > 0 ? max(0, base + q0 - window + 1) : 0);
+  const int last = DEC ? qp : base + min(q0 + 63, ql - 1);
+  int pg0 = first / PAGE_TOK, pg1 = last / PAGE_TOK + 1;
+  if constexpr (DEC) {
+    const int per = (pg1 - pg0 + nsplit - 1) / nsplit;
+    pg0 += blockIdx.x * per;
+    pg1 = min(pg1, pg0 + per);
+  }
   float m = -INFINITY, l = 0.0f;
-  if (sink) {
-    m = sink[h] * LOG2E_F;
+  if (sink && (!DEC || blockIdx.x == 0)) {
+    m = sink[head] * LOG2E_F;
     l = g == 0 ? 1.0f : 0.0f;
   }
   f32x4 acc[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  const int first = window > 0 ? max(0, base + q0 - window + 1) : 0;
-  const int last = base + min(q0 + 63, ql - 1);
   const int kchunks = DK >> 3;
-  for (int pg = first / PAGE_TOK; pg <= last / PAGE_TOK; ++pg) {
-    __syncthreads();  // the previous page's readers are done (first pass: the queries are written)
+  const int q4 = lq >> 2, p4 = lq & 3;
+  for (int pg = pg0; pg < pg1; ++pg) {
+    __syncthreads();  // the previous page's readers are done
     const uint16_t* src = cache + (int64_t)bt[pg] * PAGE_TOK * DK;
-    for (int idx = tid; idx < 64 * kchunks; idx += 256) {
+    for (int idx = tid; idx < 64 * kchunks; idx += NT) {
       const int row = idx / kchunks, dim = (idx - row * kchunks) << 3;
-      const s16x8 v = ld16(src + row * DK + dim);
-      st16(Ks + row * LDK + dim, v);
-      if (dim < R) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(dim + e) * LDV + row] = (uint16_t)v[e];
-      }
+      st16(Ks + row * LDK + dim, ld16(src + row * DK + dim));
     }
     __syncthreads();
     const int k0 = pg * PAGE_TOK;
-    // scores of the page's four 16-key sub-tiles that some query of this wave sees
+    // scores of the page's four 16-key sub-tiles that some column of this wave sees
     f32x4 S[4];
     bool live[4];
     float mx = -INFINITY;
@@ -362,8 +416,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       S[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
       if (!live[sub]) continue;
       const uint16_t* ka = Ks + (16 * sub + lq) * LDK + 8 * g;
-      const uint16_t* qb = Qs + (16 * wave + lq) * LDK + 8 * g;
-      for (int kk = 0; kk < DKp; kk += 32) S[sub] = mfma16(ld16(ka + kk), ld16(qb + kk), S[sub]);
+#pragma unroll
+      for (int i = 0; i < NQ; ++i)
+        if (i < nq) S[sub] = mfma16(ld16(ka + 32 * i), qreg[i], S[sub]);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kp = ks + 4 * g + r;
@@ -396,11 +451,13 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       if (!live[2 * kk] && !live[2 * kk + 1]) continue;
+      // V^T fragments by transposed LDS reads: lane 4 q4 + p4 of group g addresses key 32 kk (+ 16) + 4 g + q4, dims
+      // 16 i + 4 p4 .. + 3; lane lq receives dim 16 i + lq of those four keys
+      const uint16_t* vb = Ks + (32 * kk + 4 * g + q4) * LDK + 4 * p4;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         if (i >= nv) continue;
-        const uint16_t* va = Vt + (16 * i + lq) * LDV + 32 * kk + 4 * g;
-        const s16x4 a0 = *reinterpret_cast<const s16x4*>(va), a1 = *reinterpret_cast<const s16x4*>(va + 16);
+        const s16x4 a0 = tr_read(vb + 16 * i), a1 = tr_read(vb + 16 * LDK + 16 * i);
         const s16x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
         acc[i] = mfma16(a, pb[kk], acc[i]);
       }
@@ -409,8 +466,22 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!valid) return;
+  if (DEC && nsplit > 1) {
+    float* pr = part + (((int64_t)tok * H + head) * nsplit + blockIdx.x) * (2 + R);
+    if (g == 0) {
+      pr[0] = m;
+      pr[1] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (i >= nv) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pr[2 + 16 * i + 4 * g + r] = acc[i][r];
+    }
+    return;
+  }
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-  uint16_t* orow = out + ((int64_t)h * T + t0 + qi) * R;
+  uint16_t* orow = out + ((int64_t)head * T + (DEC ? tok : t0 + qi)) * R;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     if (i >= nv) continue;
@@ -418,6 +489,30 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
 #pragma unroll
     for (int r = 0; r < 4; ++r) o[r] = (short)f2bf(acc[i][r] * inv);
     *reinterpret_cast<s16x4*>(orow + 16 * i + 4 * g) = o;
+  }
+}
+
+// partials of the key splits [T, H, nsplit, 2 + R] (base-2 maximum, denominator, sums) -> out [H, T, R]
+__global__ __launch_bounds__(256) void latent_attn_merge_k(const float* __restrict__ part, int nsplit, int T, int H, int R,
+                                                          uint16_t* __restrict__ out) {
+  const int64_t th = blockIdx.x;  // t * H + h
+  const int t = (int)(th / H), h = (int)(th - (int64_t)t * H);
+  const float* p = part + th * nsplit * (2 + R);
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, p[s * (2 + R)]);
+  float L = 0.0f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = p[s * (2 + R)];
+    if (ms != -INFINITY) L += p[s * (2 + R) + 1] * exp2f(ms - M);
+  }
+  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  for (int i = threadIdx.x; i < R; i += blockDim.x) {
+    float a = 0.0f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = p[s * (2 + R)];
+      if (ms != -INFINITY) a += p[s * (2 + R) + 2 + i] * exp2f(ms - M);
+    }
+    out[((int64_t)h * T + t) * R + i] = f2bf(a * inv);
   }
 }
 
@@ -549,19 +644,19 @@ void launch_latt(dim3 grid, size_t lds, const at::Tensor& q_lat, const at::Tenso
       (AT*)out.data_ptr(), H, R, dr);
 }
 
-template <int NV>
+template <int NV, bool DEC>
 void launch_latt_mfma(dim3 grid, size_t lds, const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tensor& cache,
                       const at::Tensor& bt, const at::Tensor& cu_q, const at::Tensor& ctx, const float* sink, float scale,
-                      int window, at::Tensor& out, int H, int R, int dr) {
-  auto kern = latent_attn_mfma_k<NV>;
+                      int window, at::Tensor& out, float* part, int nsplit, int H, int R, int dr) {
+  auto kern = latent_attn_mfma_k<NV, DEC>;
   if (lds > 64 * 1024) {
     static bool attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)attr;
   }
-  kern<<<grid, 256, lds, stream()>>>(
+  kern<<<grid, DEC ? 64 : 256, lds, stream()>>>(
       (const uint16_t*)q_lat.data_ptr(), (const uint16_t*)q_pe.data_ptr(), (const uint16_t*)cache.data_ptr(),
-      bt.data_ptr<int>(), (int)bt.size(1), cu_q.data_ptr<int>(), ctx.data_ptr<int>(), (int)q_lat.size(1), sink,
-      scale * LOG2E_F, window, (uint16_t*)out.data_ptr(), H, R, dr);
+      bt.data_ptr<int>(), (int)bt.size(1), cu_q.data_ptr<int>(), ctx.data_ptr<int>(), (int)ctx.numel(), (int)q_lat.size(1),
+      sink, scale * LOG2E_F, window, (uint16_t*)out.data_ptr(), part, nsplit, H, R, dr);
 }
 
 void latent_attn(const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tensor& cache, const at::Tensor& block_tables,
@@ -592,16 +687,42 @@ void latent_attn(const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tens
   }
   const int d = (int)(R + dr);
   // (block tables, cu_q and ctx_lens come from the runner: tables cover ctx_lens, cu_q[B] == T)
-  if (LATT_MFMA && dt == at::kBFloat16 && max_qlen >= 16 && R % 16 == 0 && dr % 8 == 0 && R <= 256) {
+  // matrix-core kernels (bf16, sizes in whole MFMA tiles): prompt portions of 16 tokens and more, and steps of single
+  // tokens (a workgroup per token, block of 16 heads and share of the pages; the shares are merged afterwards)
+  if (LATT_MFMA && dt == at::kBFloat16 && (max_qlen >= 16 || max_qlen == 1) && R % 16 == 0 && dr % 8 == 0 && R <= 256) {
     const int DKp = (d + 31) & ~31;
-    const size_t lds = ((size_t)2 * 64 * (DKp + LM_PAD) + (size_t)R * (PAGE_TOK + LM_PAD)) * 2;
-    if (lds <= 160 * 1024) {
-      const dim3 grid((unsigned)((max_qlen + 63) / 64), (unsigned)B, (unsigned)H);
-      const int nv = (int)(R / 16);
-#define XOT_LM(NV) launch_latt_mfma<NV>(grid, lds, q_lat, q_pe, cache, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, out, (int)H, (int)R, (int)dr)
-      if (nv <= 4) XOT_LM(4);
-      else if (nv <= 8) XOT_LM(8);
-      else XOT_LM(16);
+    const int nv = (int)(R / 16), nq = DKp / 32;
+    const int NVT = (nv <= 4 && nq <= 4) ? 4 : ((nv <= 8 && nq <= 6) ? 8 : 16);
+    const bool dec = max_qlen == 1;
+    const size_t lds = (size_t)(dec ? 80 : 128) * (DKp + LM_PAD) * 2;
+    if (nq <= NVT / 2 + 2 && lds <= 160 * 1024) {
+      dim3 grid((unsigned)((max_qlen + 63) / 64), (unsigned)B, (unsigned)H);
+      int nsplit = 1;
+      float* part = nullptr;
+      at::Tensor ws;
+      if (dec) {
+        const int64_t hb = (H + 15) / 16, units = T * hb;
+        int64_t pages = block_tables.size(1);
+        if (window > 0) pages = std::min<int64_t>(pages, window / PAGE_TOK + 2);
+        nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(pages, 64), (768 + units - 1) / units));
+        if (nsplit > 1) {
+          ws = at::empty({T * H * nsplit * (2 + R)}, q_lat.options().dtype(at::kFloat));
+          part = ws.data_ptr<float>();
+        }
+        grid = dim3((unsigned)nsplit, (unsigned)hb, (unsigned)T);
+      }
+#define XOT_LM(NV, DEC) launch_latt_mfma<NV, DEC>(grid, lds, q_lat, q_pe, cache, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, out, part, nsplit, (int)H, (int)R, (int)dr)
+      if (dec) {
+        if (NVT == 4) XOT_LM(4, true);
+        else if (NVT == 8) XOT_LM(8, true);
+        else XOT_LM(16, true);
+        if (nsplit > 1)
+          latent_attn_merge_k<<<(unsigned)(T * H), 256, 0, stream()>>>(part, nsplit, (int)T, (int)H, (int)R, (uint16_t*)out.data_ptr());
+      } else {
+        if (NVT == 4) XOT_LM(4, false);
+        else if (NVT == 8) XOT_LM(8, false);
+        else XOT_LM(16, false);
+      }
 #undef XOT_LM
       return;
     }
