@@ -305,17 +305,17 @@ __global__ __launch_bounds__(64 * LATT_WAVES) void latent_attn_k(
 constexpr int LM_PAD = 8;
 
 template <int NV, bool DEC>
-__global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
+__global__ __launch_bounds__(256) void latent_attn_mfma_k(
     const uint16_t* __restrict__ q_lat, const uint16_t* __restrict__ q_pe, const uint16_t* __restrict__ cache,
     const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int B,
     int T, const float* __restrict__ sink, float scale_l2, int window, uint16_t* __restrict__ out, float* __restrict__ part,
     int nsplit, int H, int R, int dr) {
-  constexpr int NQ = NV / 2 + 2, NT = DEC ? 64 : 256, QROWS = DEC ? 16 : 64;
+  constexpr int NQ = NV / 2 + 2, NT = 256, QROWS = DEC ? 16 : 64;
   extern __shared__ __attribute__((aligned(16))) uint16_t lsm[];
   const int DK = R + dr, DKp = (DK + 31) & ~31, LDK = DKp + LM_PAD;
   const int nv = R >> 4, nq = DKp >> 5;
   uint16_t* Qs = lsm;                 // [QROWS][LDK]
-  uint16_t* Ks = Qs + QROWS * LDK;    // [64][LDK]
+  uint16_t* Ks = Qs + QROWS * LDK;    // [2][64][LDK]: the page in use and the next one
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, lq = lane & 15;
   int b, h0 = 0, t0 = 0, ql = 0, q0 = 0, base = 0, tok = 0;
   if constexpr (DEC) {
@@ -334,7 +334,7 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
   const int head = DEC ? min(h0 + lq, H - 1) : h0;
   if constexpr (DEC) {
     if (n <= 0) {  // padding row of a captured decode batch: zeros, an empty partial
-      if (h0 + lq < H) {
+      if (h0 + lq < H && wave == 0) {
         if (nsplit == 1) {
           for (int i = g; i < R; i += 4) out[((int64_t)head * T + tok) * R + i] = 0;
         } else {
@@ -361,7 +361,7 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
     }
     st16(Qs + row * LDK + dim, v);
   }
-  for (int idx = tid; idx < 64 * ((DKp - DK) >> 3); idx += NT) {  // the keys' padding columns stay zero
+  for (int idx = tid; idx < 128 * ((DKp - DK) >> 3); idx += NT) {  // the keys' padding columns stay zero
     const int pc = (DKp - DK) >> 3, row = idx / pc, dim = DK + ((idx - row * pc) << 3);
     st16(Ks + row * LDK + dim, s16x8{0, 0, 0, 0, 0, 0, 0, 0});
   }
@@ -396,14 +396,40 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
   for (int i = 0; i < NV; ++i) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   const int kchunks = DK >> 3;
   const int q4 = lq >> 2, p4 = lq & 3;
-  for (int pg = pg0; pg < pg1; ++pg) {
-    __syncthreads();  // the previous page's readers are done
+  // a page's rows travel global -> registers -> LDS, a thread's chunks all in flight at once; the next page is
+  // fetched into registers before this page's MFMAs and written to the other buffer after them
+  s16x8 pre[NQ];
+  auto fetch = [&](int pg) {
     const uint16_t* src = cache + (int64_t)bt[pg] * PAGE_TOK * DK;
-    for (int idx = tid; idx < 64 * kchunks; idx += NT) {
-      const int row = idx / kchunks, dim = (idx - row * kchunks) << 3;
-      st16(Ks + row * LDK + dim, ld16(src + row * DK + dim));
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int idx = tid + NT * u;
+      if (idx < 64 * kchunks) {
+        const int row = idx / kchunks, dim = (idx - row * kchunks) << 3;
+        pre[u] = ld16(src + row * DK + dim);
+      }
     }
-    __syncthreads();
+  };
+  auto commit = [&](uint16_t* dst) {
+#pragma unroll
+    for (int u = 0; u < NQ; ++u) {
+      const int idx = tid + NT * u;
+      if (idx < 64 * kchunks) {
+        const int row = idx / kchunks, dim = (idx - row * kchunks) << 3;
+        st16(dst + row * LDK + dim, pre[u]);
+      }
+    }
+  };
+  if (pg0 < pg1) {
+    fetch(pg0);
+    commit(Ks);
+  }
+  __syncthreads();
+  for (int pg = pg0; pg < pg1; ++pg) {
+    const uint16_t* Kc = Ks + ((pg - pg0) & 1) * 64 * LDK;
+    const bool more = pg + 1 < pg1;
+    if (more) fetch(pg + 1);
+    if (!DEC || wave == 0) {
     const int k0 = pg * PAGE_TOK;
     // scores of the page's four 16-key sub-tiles that some column of this wave sees
     f32x4 S[4];
@@ -415,7 +441,7 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
       live[sub] = ks <= wq_hi && (window == 0 || ks + 15 > wq_lo - window) && wq_lo <= wq_hi;
       S[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
       if (!live[sub]) continue;
-      const uint16_t* ka = Ks + (16 * sub + lq) * LDK + 8 * g;
+      const uint16_t* ka = Kc + (16 * sub + lq) * LDK + 8 * g;
 #pragma unroll
       for (int i = 0; i < NQ; ++i)
         if (i < nq) S[sub] = mfma16(ld16(ka + 32 * i), qreg[i], S[sub]);
@@ -453,7 +479,7 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
       if (!live[2 * kk] && !live[2 * kk + 1]) continue;
       // V^T fragments by transposed LDS reads: lane 4 q4 + p4 of group g addresses key 32 kk (+ 16) + 4 g + q4, dims
       // 16 i + 4 p4 .. + 3; lane lq receives dim 16 i + lq of those four keys
-      const uint16_t* vb = Ks + (32 * kk + 4 * g + q4) * LDK + 4 * p4;
+      const uint16_t* vb = Kc + (32 * kk + 4 * g + q4) * LDK + 4 * p4;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         if (i >= nv) continue;
@@ -462,7 +488,11 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
         acc[i] = mfma16(a, pb[kk], acc[i]);
       }
     }
+    }
+    if (more) commit(Ks + (((pg - pg0) & 1) ^ 1) * 64 * LDK);
+    __syncthreads();  // the next page is written, this one's readers are done
   }
+  if (DEC && wave != 0) return;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!valid) return;
@@ -495,24 +525,25 @@ __global__ __launch_bounds__(DEC ? 64 : 256) void latent_attn_mfma_k(
 // partials of the key splits [T, H, nsplit, 2 + R] (base-2 maximum, denominator, sums) -> out [H, T, R]
 __global__ __launch_bounds__(256) void latent_attn_merge_k(const float* __restrict__ part, int nsplit, int T, int H, int R,
                                                           uint16_t* __restrict__ out) {
+  __shared__ float w[64];  // nsplit <= 64: the first wave weighs the splits
   const int64_t th = blockIdx.x;  // t * H + h
   const int t = (int)(th / H), h = (int)(th - (int64_t)t * H);
   const float* p = part + th * nsplit * (2 + R);
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, p[s * (2 + R)]);
-  float L = 0.0f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = p[s * (2 + R)];
-    if (ms != -INFINITY) L += p[s * (2 + R) + 1] * exp2f(ms - M);
+  if (threadIdx.x < 64) {
+    const int sidx = threadIdx.x;
+    const float ms = sidx < nsplit ? p[sidx * (2 + R)] : -INFINITY;
+    const float ls = sidx < nsplit ? p[sidx * (2 + R) + 1] : 0.0f;
+    const float M = wave_max(ms);
+    const float f = ms == -INFINITY ? 0.0f : exp2f(ms - M);
+    const float L = wave_sum(ls * f);
+    w[sidx] = L > 0.0f ? f / L : 0.0f;
   }
-  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  __syncthreads();
   for (int i = threadIdx.x; i < R; i += blockDim.x) {
     float a = 0.0f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float ms = p[s * (2 + R)];
-      if (ms != -INFINITY) a += p[s * (2 + R) + 2 + i] * exp2f(ms - M);
-    }
-    out[((int64_t)h * T + t) * R + i] = f2bf(a * inv);
+#pragma unroll 4
+    for (int sp = 0; sp < nsplit; ++sp) a += w[sp] * p[sp * (2 + R) + 2 + i];
+    out[((int64_t)h * T + t) * R + i] = f2bf(a);
   }
 }
 
@@ -653,7 +684,7 @@ void launch_latt_mfma(dim3 grid, size_t lds, const at::Tensor& q_lat, const at::
     static bool attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)attr;
   }
-  kern<<<grid, DEC ? 64 : 256, lds, stream()>>>(
+  kern<<<grid, 256, lds, stream()>>>(
       (const uint16_t*)q_lat.data_ptr(), (const uint16_t*)q_pe.data_ptr(), (const uint16_t*)cache.data_ptr(),
       bt.data_ptr<int>(), (int)bt.size(1), cu_q.data_ptr<int>(), ctx.data_ptr<int>(), (int)ctx.numel(), (int)q_lat.size(1),
       sink, scale * LOG2E_F, window, (uint16_t*)out.data_ptr(), part, nsplit, H, R, dr);
@@ -694,7 +725,7 @@ void latent_attn(const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tens
     const int nv = (int)(R / 16), nq = DKp / 32;
     const int NVT = (nv <= 4 && nq <= 4) ? 4 : ((nv <= 8 && nq <= 6) ? 8 : 16);
     const bool dec = max_qlen == 1;
-    const size_t lds = (size_t)(dec ? 80 : 128) * (DKp + LM_PAD) * 2;
+    const size_t lds = (size_t)(dec ? 144 : 192) * (DKp + LM_PAD) * 2;
     if (nq <= NVT / 2 + 2 && lds <= 160 * 1024) {
       dim3 grid((unsigned)((max_qlen + 63) / 64), (unsigned)B, (unsigned)H);
       int nsplit = 1;
@@ -704,7 +735,7 @@ void latent_attn(const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tens
         const int64_t hb = (H + 15) / 16, units = T * hb;
         int64_t pages = block_tables.size(1);
         if (window > 0) pages = std::min<int64_t>(pages, window / PAGE_TOK + 2);
-        nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(pages, 64), (768 + units - 1) / units));
+        nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(pages, 64), (256 + units - 1) / units));
         if (nsplit > 1) {
           ws = at::empty({T * H * nsplit * (2 + R)}, q_lat.options().dtype(at::kFloat));
           part = ws.data_ptr<float>();
