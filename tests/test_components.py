@@ -41,7 +41,7 @@ def test_presets_match_hf_shapes():
   assert (c.num_layers, c.hidden_size, c.num_heads, c.num_kv_heads, c.intermediate_size, c.vocab_size) == \
          (80, 8192, 64, 8, 28672, 128256)
   for name, cfg in PRESETS.items():
-    assert cfg.is_mla or cfg.hidden_size == cfg.num_heads * cfg.head_dim or cfg.head_dim in (64, 128), name
+    assert cfg.is_mla or cfg.is_mixed or cfg.hidden_size == cfg.num_heads * cfg.head_dim or cfg.head_dim in (64, 128), name
   # every model card with a preset agrees on the layer count; parameter totals of the big dense cards
   for name, card in R.model_cards.items():
     if name in PRESETS:
