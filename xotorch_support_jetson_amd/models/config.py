@@ -349,7 +349,8 @@ class ModelConfig:
   def with_layers(self, n: int) -> "ModelConfig":
     if self.layer_specs is not None and n != len(self.layer_specs):
       specs = tuple(self.layer_specs[i % len(self.layer_specs)] for i in range(n))
-      return replace(self, num_layers=n, layer_specs=specs)
+      loop = self.loop if self.loop and self.loop[1] <= n else None  # (a loop that no longer fits is dropped)
+      return replace(self, num_layers=n, layer_specs=specs, loop=loop)
     return replace(self, num_layers=n)
 
 
