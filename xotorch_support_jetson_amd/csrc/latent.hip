@@ -310,10 +310,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int B,
     int T, const float* __restrict__ sink, float scale_l2, int window, uint16_t* __restrict__ out, float* __restrict__ part,
     int nsplit, int H, int R, int dr) {
-  constexpr int NQ = NV / 2 + 2, NT = 256, QROWS = DEC ? 16 : 64;
+  // (row length and output tiles are the template's bounds: columns past the real sizes hold zeros, output tiles past
+  // the latent are computed and dropped, so the MFMA loops have no run-time conditions and pipeline their LDS reads)
+  constexpr int NQ = NV / 2 + 2, NT = 256, QROWS = DEC ? 16 : 64, DKp = NQ * 32, LDK = DKp + LM_PAD;
   extern __shared__ __attribute__((aligned(16))) uint16_t lsm[];
-  const int DK = R + dr, DKp = (DK + 31) & ~31, LDK = DKp + LM_PAD;
-  const int nv = R >> 4, nq = DKp >> 5;
+  const int DK = R + dr, nv = R >> 4;
   uint16_t* Qs = lsm;                 // [QROWS][LDK]
   uint16_t* Ks = Qs + QROWS * LDK;    // [2][64][LDK]: the page in use and the next one
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, lq = lane & 15;
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
   if constexpr (DEC) {
     tok = blockIdx.z;
     h0 = blockIdx.y * 16;
-    b = seq_of(cu_q, B, tok);
+    b = tok;  // (a step of single tokens: token t is sequence t's)
   } else {
     b = blockIdx.y;
     h0 = blockIdx.z;
@@ -348,30 +349,6 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
     if (n <= 0 || q0 >= ql) return;
   }
   const int* bt = block_tables + (int64_t)b * width;
-  // queries -> LDS (rows without a query and the padding columns: zero), then into registers as B operands
-  const int chunks = DKp >> 3;
-  for (int idx = tid; idx < QROWS * chunks; idx += NT) {
-    const int row = idx / chunks, dim = (idx - row * chunks) << 3;
-    s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bool has = DEC ? (h0 + row < H) : (q0 + row < ql);
-    if (has && dim < DK) {
-      const int64_t t = DEC ? tok : t0 + q0 + row;
-      const int hh = DEC ? h0 + row : h0;
-      v = dim < R ? ld16(q_lat + ((int64_t)hh * T + t) * R + dim) : ld16(q_pe + (t * H + hh) * dr + (dim - R));
-    }
-    st16(Qs + row * LDK + dim, v);
-  }
-  for (int idx = tid; idx < 128 * ((DKp - DK) >> 3); idx += NT) {  // the keys' padding columns stay zero
-    const int pc = (DKp - DK) >> 3, row = idx / pc, dim = DK + ((idx - row * pc) << 3);
-    st16(Ks + row * LDK + dim, s16x8{0, 0, 0, 0, 0, 0, 0, 0});
-  }
-  __syncthreads();
-  s16x8 qreg[NQ];
-  {
-    const uint16_t* qb = Qs + ((DEC ? 0 : 16 * wave) + lq) * LDK + 8 * g;
-#pragma unroll
-    for (int i = 0; i < NQ; ++i) qreg[i] = i < nq ? ld16(qb + 32 * i) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
-  }
   // this lane's column: its query's position, whether it is a real one
   const int qi = DEC ? 0 : q0 + 16 * wave + lq;
   const bool valid = DEC ? (h0 + lq < H) : (qi < ql);
@@ -420,11 +397,32 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       }
     }
   };
-  if (pg0 < pg1) {
-    fetch(pg0);
-    commit(Ks);
+  if (pg0 < pg1) fetch(pg0);  // (in flight while the queries are staged)
+  // queries -> LDS (rows without a query and the padding columns: zero), then into registers as B operands
+  const int chunks = DKp >> 3;
+  for (int idx = tid; idx < QROWS * chunks; idx += NT) {
+    const int row = idx / chunks, dim = (idx - row * chunks) << 3;
+    s16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool has = DEC ? (h0 + row < H) : (q0 + row < ql);
+    if (has && dim < DK) {
+      const int64_t t = DEC ? tok : t0 + q0 + row;
+      const int hh = DEC ? h0 + row : h0;
+      v = dim < R ? ld16(q_lat + ((int64_t)hh * T + t) * R + dim) : ld16(q_pe + (t * H + hh) * dr + (dim - R));
+    }
+    st16(Qs + row * LDK + dim, v);
   }
+  for (int idx = tid; idx < 128 * ((DKp - DK) >> 3); idx += NT) {  // the keys' padding columns stay zero
+    const int pc = (DKp - DK) >> 3, row = idx / pc, dim = DK + ((idx - row * pc) << 3);
+    st16(Ks + row * LDK + dim, s16x8{0, 0, 0, 0, 0, 0, 0, 0});
+  }
+  if (pg0 < pg1) commit(Ks);
   __syncthreads();
+  s16x8 qreg[NQ];
+  {
+    const uint16_t* qb = Qs + ((DEC ? 0 : 16 * wave) + lq) * LDK + 8 * g;
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) qreg[i] = ld16(qb + 32 * i);
+  }
   for (int pg = pg0; pg < pg1; ++pg) {
     const uint16_t* Kc = Ks + ((pg - pg0) & 1) * 64 * LDK;
     const bool more = pg + 1 < pg1;
@@ -443,8 +441,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       if (!live[sub]) continue;
       const uint16_t* ka = Kc + (16 * sub + lq) * LDK + 8 * g;
 #pragma unroll
-      for (int i = 0; i < NQ; ++i)
-        if (i < nq) S[sub] = mfma16(ld16(ka + 32 * i), qreg[i], S[sub]);
+      for (int i = 0; i < NQ; ++i) S[sub] = mfma16(ld16(ka + 32 * i), qreg[i], S[sub]);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kp = ks + 4 * g + r;
@@ -472,8 +469,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       }
     l = l * corr + ls;
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-      if (i < nv) acc[i] *= corr;
+    for (int i = 0; i < NV; ++i) acc[i] *= corr;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       if (!live[2 * kk] && !live[2 * kk + 1]) continue;
@@ -482,7 +478,6 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_k(
       const uint16_t* vb = Kc + (32 * kk + 4 * g + q4) * LDK + 4 * p4;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        if (i >= nv) continue;
         const s16x4 a0 = tr_read(vb + 16 * i), a1 = tr_read(vb + 16 * LDK + 16 * i);
         const s16x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
         acc[i] = mfma16(a, pb[kk], acc[i]);
@@ -721,12 +716,11 @@ void latent_attn(const at::Tensor& q_lat, const at::Tensor& q_pe, const at::Tens
   // matrix-core kernels (bf16, sizes in whole MFMA tiles): prompt portions of 16 tokens and more, and steps of single
   // tokens (a workgroup per token, block of 16 heads and share of the pages; the shares are merged afterwards)
   if (LATT_MFMA && dt == at::kBFloat16 && (max_qlen >= 16 || max_qlen == 1) && R % 16 == 0 && dr % 8 == 0 && R <= 256) {
-    const int DKp = (d + 31) & ~31;
-    const int nv = (int)(R / 16), nq = DKp / 32;
+    const int nv = (int)(R / 16), nq = (d + 31) / 32;
     const int NVT = (nv <= 4 && nq <= 4) ? 4 : ((nv <= 8 && nq <= 6) ? 8 : 16);
     const bool dec = max_qlen == 1;
-    const size_t lds = (size_t)(dec ? 144 : 192) * (DKp + LM_PAD) * 2;
-    if (nq <= NVT / 2 + 2 && lds <= 160 * 1024) {
+    const size_t lds = (size_t)(dec ? 144 : 192) * ((NVT / 2 + 2) * 32 + LM_PAD) * 2;
+    if (nq <= NVT / 2 + 2 && lds <= 160 * 1024 && (!dec || T == B)) {
       dim3 grid((unsigned)((max_qlen + 63) / 64), (unsigned)B, (unsigned)H);
       int nsplit = 1;
       float* part = nullptr;
