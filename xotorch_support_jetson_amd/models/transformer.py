@@ -744,10 +744,8 @@ class ShardModel:
       S = S_dn if big else (4 if T * k <= 64 else 2)
       if Fp % (256 * S):
         S = 1
-      gu = torch.empty(T * k, 2 * Fp, dtype=torch.float32, device=dev)
-      C.gemm_moe(hn, lw.ex_up_w, gu, off, sorted_tok, K.EPI["none"], T, sh_up, 1, bm)
-      act = torch.empty(T * k, Fp, dtype=torch.bfloat16, device=dev)
-      K.glu_act(gu, 0, Fp, Fp, False, 0.0, act)
+      act = torch.empty(T * k, Fp, dtype=torch.bfloat16, device=dev)  # silu(gate) * up in the GEMM's epilogue
+      C.gemm_moe(hn, lw.ex_up_w, act, off, sorted_tok, K.EPI["silu"], T, sh_up, 1, bm)
       y = torch.empty(S * T * k, Dq, dtype=torch.float32, device=dev)
       C.gemm_moe(act, lw.ex_down_w, y, off, None, K.EPI["none"], T, sh_dn, S, bm_dn)
     else:
@@ -757,8 +755,9 @@ class ShardModel:
       for e in range(E):
         if offs[e + 1] > offs[e]:
           xe = hn.index_select(0, sorted_tok[offs[e]:offs[e + 1]].long()).float()
-          gu = xe @ lw.ex_up_w[e].float().t()
-          y[offs[e]:offs[e + 1]] = (torch.nn.functional.silu(gu[:, :Fp]) * gu[:, Fp:]) @ lw.ex_down_w[e].float().t()
+          gu = (xe @ lw.ex_up_w[e].float().t()).reshape(xe.shape[0], Fp // 16, 2, 16)  # (gate | up tiles of 16)
+          act = (torch.nn.functional.silu(gu[:, :, 0]) * gu[:, :, 1]).reshape(xe.shape[0], Fp)
+          y[offs[e]:offs[e + 1]] = act @ lw.ex_down_w[e].float().t()
     sh_y = None
     if f.shared_ff:
       act = rows("sh_act", f.shared_ff, lw.down_w.shape[1])

@@ -721,7 +721,7 @@ class MixedLayerWeights:
   ff_cols: Optional[Dict[str, tuple]] = None
   act: Optional[torch.Tensor] = None  # [4] fp32 PolyNorm coefficients
   router_b: Optional[torch.Tensor] = None  # [E] fp32
-  ex_up_w: Optional[torch.Tensor] = None  # [E, Fp, Dp] experts' up projections ([E, 2 Fp, Dp]: gate rows, then up rows)
+  ex_up_w: Optional[torch.Tensor] = None  # [E, Fp, Dp] experts' up projections ([E, 2 Fp, Dp]: gate / up rows interleaved by 16)
   ex_down_w: Optional[torch.Tensor] = None  # [E, Dq, Fp]
   # sandwich blocks (config.block "sandwich"): norm1 / norm2 weigh the sublayers' inputs, norm1b / norm2b their
   # results; latent attention: `in_w` = [q (or the query latent) | kv latent | rotated key part | output gate]
@@ -902,7 +902,8 @@ def build_sandwich_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayer
       fb += [("sh_gate", get(q + "shared.gate")), ("sh_up", get(q + "shared.up"))]
       down = get(q + "shared.down")
     Fp, Dp = _up(f.ff, 128), _up(D, 128)
-    lw.ex_up_w = dev(torch.stack([torch.cat([_pad2(get(q + f"e{e}.gate"), Fp, Dp), _pad2(get(q + f"e{e}.up"), Fp, Dp)])
+    # gate and up rows interleaved in tiles of 16 (the grouped GEMM's SiLU epilogue pairs them)
+    lw.ex_up_w = dev(torch.stack([interleave_gate_up(_pad2(get(q + f"e{e}.gate"), Fp, Dp), _pad2(get(q + f"e{e}.up"), Fp, Dp))
                                   for e in range(f.experts)]), dtype)
     lw.ex_down_w = dev(torch.stack([_pad2(get(q + f"e{e}.down"), Dp, Fp) for e in range(f.experts)]), dtype)
   ff_w, lw.ff_cols = _fused_rows(fb, D)
