@@ -37,8 +37,14 @@ class LinearRecurrenceSpec:
   rule "delta": scalar decay per head g = exp(-exp(A_log) softplus(a + dt_bias)), write k (beta (v - S^T k))^T,
     q / k shared by heads / kv_heads value heads, short causal convolutions (conv taps) + SiLU on q, k, v,
     unit-norm q and k, q scaled by dim^-1/2.
-  rule "gla": decay per key channel sigmoid(z)^(1/tau) with a low-rank z, write k v^T, q scaled by dim^-1/2."""
-  rule: str  # delta | gla
+  rule "gla": decay per key channel sigmoid(z)^(1/tau) with a low-rank z, write k v^T, q scaled by dim^-1/2.
+  rule "lightning": one fixed decay per head (`decays`), SiLU on q, k, v, write k v^T, no scale; the heads' outputs are
+    RMS-normed together, weighted and gated by a sigmoid.
+  rule "mlstm": the matrix memory of xLSTM.  Log input gate i = cap tanh(z_i / cap), log forget gate f = logsigmoid(cap
+    tanh(z_f / cap)) per head (gate_cap), a running maximum m_t = max(f + m_(t-1), i) that starts at 0, S <- e^(f + m_(t-1) -
+    m_t) S + e^(i - m_t) k v^T and a normaliser n likewise from k alone, o = S^T q / (max(|n . q|, e^(-m_t)) + 1e-6), q
+    scaled by dim^-1/2.  The normaliser travels as one more value channel of the state (value = 1), the maximum beside it."""
+  rule: str  # delta | gla | lightning | mlstm
   heads: int
   kv_heads: int
   dim: int
@@ -46,6 +52,13 @@ class LinearRecurrenceSpec:
   conv: int = 0  # taps of the short convolutions (delta)
   tau: float = 1.0  # decay temperature (gla)
   rank: int = 0  # rank of the decay projection (gla; from the tensor's shape)
+  decays: tuple = ()  # lightning: one per head
+  gate_cap: float = 0.0  # mlstm
+
+  @property
+  def state_vdim(self) -> int:
+    """Value channels of the state: mlstm keeps its normaliser as one channel more."""
+    return self.vdim + 1 if self.rule == "mlstm" else self.vdim
 
 
 @dataclass(frozen=True)
@@ -56,7 +69,8 @@ class WindowAttnSpec:
   one softmax.  q / k / v may carry biases; rotate-half RoPE on the first rot_dims dims with optional wavelength-banded
   frequency scaling rot_scaling = (factor, low, high, original); qk_norm divides q and k by their RMS per head after
   the rotation.  kv_from >= 0: no key / value projections, the layer reads that layer's caches with its own queries
-  and its own window / pool."""
+  and its own window / pool.  gate "elem": the heads' outputs times sigmoid of a projection of the mixer's input, element
+  by element."""
   heads: int
   kv_heads: int
   dim: int
@@ -71,6 +85,25 @@ class WindowAttnSpec:
   bias: bool = True
   sink: bool = True
   kv_from: int = -1
+  gate: str = "none"  # none | elem
+
+
+@dataclass(frozen=True)
+class DiffAttnSpec:
+  """Differential softmax attention (GQA): every head holds two query / key maps of size dim that attend to the same
+  values; o = a_1 - lam a_2 with lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init (learned vectors, one number per
+  layer), then o / rms(o) per head (no weight) times (1 - lam_init), times sigmoid of one gate per head.  RoPE on the
+  first rot_dims dims of each map, pairs (2i, 2i + 1); window > 0: a query at position i sees 0 <= i - j < window, else
+  every j <= i.  The cache holds 2 kv_heads key heads (a kv head's two maps side by side) and kv_heads value heads."""
+  heads: int
+  kv_heads: int
+  dim: int
+  vdim: int
+  window: int
+  rot_dims: int
+  rot_base: float
+  scale: float
+  lam_init: float
 
 
 @dataclass(frozen=True)
@@ -99,8 +132,8 @@ class SSDSpec:
 class FeedForwardSpec:
   """A non-gated feed-forward W_down act(W_up h).  kind "polynorm": act(z) = a N(z) + b N(z^2) + c N(z^3) + e with N the
   division of the token's ff vector by its RMS; kind "relu2_moe": `experts` experts with act = relu^2, the `top` largest
-  router logits chosen per token and weighted by the softmax over the chosen logits, plus (shared_ff > 0) one shared
-  expert of the same form scaled by a per-token sigmoid gate.
+  router logits chosen per token and weighted by the softmax over the chosen logits (or the `route` rule below), plus
+  (shared_ff > 0) one shared expert of the same form scaled by a per-token sigmoid gate.
   Gated kinds, W_down (a(W_gate h) * b(W_up h)): "clamped_glu": g = min(gate, limit), u = clamp(up, -limit, limit),
   g sigmoid(1.702 g) (u + 1); "silu_moe": `experts` SiLU-gated experts, scores = softmax of the router logits over
   all experts, the `top` largest chosen and weighted by their scores as they are (no renormalisation), plus
@@ -111,6 +144,14 @@ class FeedForwardSpec:
   top: int = 0
   shared_ff: int = 0
   limit: float = 0.0  # clamped_glu
+  # relu2_moe routing.  "softmax_top": the rule above.  "sigmoid_groups": scores = sigmoid(logits); the choice is made on
+  # scores + a learned correction, among the experts of the `keep` best of `groups` equal groups of neighbours (a
+  # group's value: the sum of its two largest corrected scores); weights = the chosen experts' uncorrected scores over
+  # their sum, times route_scale
+  route: str = "softmax_top"
+  groups: int = 1
+  keep: int = 1
+  route_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -157,13 +198,17 @@ class MixedLayerSpec:
   ssd: Optional[SSDSpec] = None
   ffn: Optional[FeedForwardSpec] = None
   lattn: Optional[LatentAttnSpec] = None  # sandwich blocks
+  dattn: Optional[DiffAttnSpec] = None  # sandwich blocks; a "parallel" layer there is wattn beside rec
 
   @property
   def kv_dims(self) -> Optional[tuple]:
-    """(kv heads, key dim, value dim) of the paged K / V pool this layer owns (None: it has none of its own).  A
-    latent-attention layer keeps one row [kv_rank | rot_dim] per token and no value pool (value dim 0)."""
+    """(key heads, key dim, value dim[, value heads]) of the paged K / V pool this layer owns (None: it has none of its
+    own).  A latent-attention layer keeps one row [kv_rank | rot_dim] per token and no value pool (value dim 0); a
+    differential-attention layer two key heads per value head."""
     if self.lattn is not None:
       return 1, self.lattn.kv_rank + self.lattn.rot_dim, 0
+    if self.dattn is not None:
+      return 2 * self.dattn.kv_heads, self.dattn.dim, self.dattn.vdim, self.dattn.kv_heads
     if self.attn is not None:
       return self.attn.kv_heads, self.attn.dim, self.attn.dim
     if self.wattn is not None and self.wattn.kv_from < 0:
@@ -172,13 +217,15 @@ class MixedLayerSpec:
 
   @property
   def state_dims(self) -> Optional[tuple]:
-    """(heads, value dim, key dim, convolution taps, convolution channels) of the layer's recurrent state."""
+    """(heads, value channels, key dim, convolution taps, convolution channels, scalars per head) of the layer's
+    recurrent state."""
     if self.rec is not None:
       r = self.rec
-      return r.heads, r.vdim, r.dim, r.conv, (2 * r.kv_heads * r.dim + r.heads * r.vdim) if r.conv > 0 else 0
+      return r.heads, r.state_vdim, r.dim, r.conv, (2 * r.kv_heads * r.dim + r.heads * r.vdim) if r.conv > 0 else 0, \
+        1 if r.rule == "mlstm" else 0
     if self.ssd is not None:
       m = self.ssd
-      return m.heads, m.vdim, m.state, m.conv, m.conv_channels if m.conv > 0 else 0
+      return m.heads, m.vdim, m.state, m.conv, m.conv_channels if m.conv > 0 else 0, 0
     return None
 
 
@@ -242,6 +289,12 @@ class ModelConfig:
   embed_scale: float = 1.0
   logit_softcap: float = 0.0  # > 0: logits <- cap * tanh(logits / cap)
   loop: Optional[tuple] = None
+  # sandwich blocks with layer norms (Kopalorn): every norm is (x - mean) / sqrt(var + eps) * w + b, the sublayers'
+  # normed results enter the stream times residual_mult, and a pass of the loop starts with x <- x + embedding output
+  # (passes after the first) + step[pass] instead of the linear mix
+  norm_kind: str = "rms"  # rms | layer
+  residual_mult: float = 1.0
+  loop_input: str = "linear"  # linear | add
 
   def layer_runs(self, layers=None) -> list:
     """[(layer, pass or -1)] in execution order for the given layers (default: all): a looped layer appears once per
@@ -354,7 +407,26 @@ class ModelConfig:
     return replace(self, num_layers=n)
 
 
+def _ln_sandwich_params(D: int, s: MixedLayerSpec) -> int:
+  """Layers of layer-norm sandwich blocks: differential attention, mlstm, or gated attention beside lightning attention."""
+  n = 4 * D  # the mixer's two norms with their biases
+  a, w, r, f = s.dattn, s.wattn, s.rec, s.ffn
+  if a is not None:
+    n += D * (2 * a.heads * a.dim + 2 * a.kv_heads * a.dim + a.kv_heads * a.vdim + a.heads) + 4 * a.dim + a.heads * a.vdim * D
+  if w is not None:
+    n += (D + 1) * (w.heads * w.dim + w.kv_heads * (w.dim + w.vdim)) + 2 * w.heads * w.vdim * D + 2 * D
+  if r is not None:
+    n += D * r.heads * (2 * r.dim + 2 * r.vdim) + r.heads * r.vdim * (D + 1)
+    if r.rule == "mlstm":
+      n += 2 * r.heads * (D + 1)
+  if f is not None:
+    n += 4 * D + f.experts * (2 * D * f.ff + D + 1) + (2 * D * f.shared_ff + D if f.shared_ff else 0)
+  return n
+
+
 def mixed_layer_params(D: int, s: MixedLayerSpec) -> int:
+  if s.dattn is not None or (s.rec is not None and s.rec.rule in ("lightning", "mlstm")):
+    return _ln_sandwich_params(D, s)
   if s.lattn is not None:
     a, f = s.lattn, s.ffn
     qd = a.heads * (a.dim + a.rot_dim)
@@ -573,7 +645,72 @@ def _nenizen_config(cfg: dict) -> ModelConfig:
     logit_softcap=float(cfg.get("logit_softcap") or 0.0), loop=loop)
 
 
+def _kopalorn_config(cfg: dict) -> ModelConfig:
+  """Kopalorn config.json: {"architecture", "vocab", "width", "norm": {"eps"}, "residual_mult", "loop": {"start", "stop",
+  "times"} | null, "layers": [{"type": "attention" | "mlstm" | "parallel", "mixer": {...}, "mlp": {"kind": "moe", "expert":
+  {"ff"}, "router": {"experts", "top", "scale", "groups": {"count", "keep"}}, "shared": {"ff"}} | null}]}.  "attention":
+  {"heads", "kv_heads", "dim", "vdim", "diff", "scale", "mask": {"size"}, "rot": {"base", "dims"}}; "mlstm": {"heads", "dim",
+  "vdim", "gate_cap"}; "parallel": {"left": {"heads", "kv_heads", "dim", "vdim", "scale"}, "right": {"heads", "dim", "vdim",
+  "decay": [one per head]}}.  Without "mask" every earlier token is seen, without "rot" nothing is rotated."""
+  specs = []
+  for i, L in enumerate(cfg["layers"]):
+    m, mlp = L["mixer"], L.get("mlp")
+    ffn = None
+    if mlp is not None:
+      if mlp.get("kind", "moe") != "moe":
+        raise ValueError(f"layer {i}: unsupported feed-forward kind {mlp.get('kind')!r}")
+      r, sh = mlp["router"], mlp.get("shared")
+      gr = r.get("groups") or {}
+      ffn = FeedForwardSpec("relu2_moe", int(mlp["expert"]["ff"]), int(r["experts"]), int(r["top"]), int(sh["ff"]) if sh else 0,
+                            route="sigmoid_groups", groups=int(gr.get("count", 1)), keep=int(gr.get("keep", gr.get("count", 1))),
+                            route_scale=float(r.get("scale", 1.0)))
+      if not 1 <= ffn.top <= ffn.experts or ffn.experts % ffn.groups or not 1 <= ffn.keep <= ffn.groups or \
+         ffn.keep * (ffn.experts // ffn.groups) < ffn.top:
+        raise ValueError(f"layer {i}: top {ffn.top} of {ffn.experts} experts in {ffn.groups} groups, {ffn.keep} kept")
+    if L["type"] == "attention":
+      rot, mask = m.get("rot") or {}, m.get("mask") or {}
+      a = DiffAttnSpec(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), int(mask.get("size", 0)),
+                       int(rot.get("dims", 0)), float(rot.get("base", 10000.0)), float(m["scale"]), float(m["diff"]))
+      if a.heads % a.kv_heads or a.rot_dims % 2 or a.rot_dims > a.dim:
+        raise ValueError(f"layer {i}: heads {a.heads} / kv_heads {a.kv_heads} / rotary dims {a.rot_dims} do not fit")
+      specs.append(MixedLayerSpec("attention", dattn=a, ffn=ffn))
+    elif L["type"] == "mlstm":
+      r = LinearRecurrenceSpec("mlstm", int(m["heads"]), int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                               gate_cap=float(m["gate_cap"]))
+      specs.append(MixedLayerSpec("mlstm", rec=r, ffn=ffn))
+    elif L["type"] == "parallel":
+      a, r = m["left"], m["right"]
+      w = WindowAttnSpec(int(a["heads"]), int(a["kv_heads"]), int(a["dim"]), int(a["vdim"]), 0, 0, 0, 10000.0, None,
+                         float(a["scale"]), qk_norm=False, bias=True, sink=False, gate="elem")
+      if w.heads % w.kv_heads:
+        raise ValueError(f"layer {i}: heads {w.heads} / kv_heads {w.kv_heads} do not fit")
+      decays = tuple(float(x) for x in r["decay"])
+      if len(decays) != int(r["heads"]):
+        raise ValueError(f"layer {i}: {len(decays)} decays for {r['heads']} heads")
+      rec = LinearRecurrenceSpec("lightning", int(r["heads"]), int(r["heads"]), int(r["dim"]), int(r["vdim"]), decays=decays)
+      specs.append(MixedLayerSpec("parallel", rec=rec, wattn=w, ffn=ffn))
+    else:
+      raise ValueError(f"layer {i}: unknown layer type {L['type']!r}")
+  lp = cfg.get("loop")
+  loop = None
+  if lp and int(lp.get("times", 1)) >= 1 and int(lp["stop"]) > int(lp["start"]):
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+    if not 0 <= loop[0] < loop[1] <= len(specs):
+      raise ValueError(f"loop {loop} outside the {len(specs)} layers")
+  first = next((s.dattn or s.wattn for s in specs if s.dattn or s.wattn), None)
+  return ModelConfig(
+    model_type="kopalorn", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+    intermediate_size=max([s.ffn.ff for s in specs if s.ffn is not None] + [0]), num_layers=len(specs),
+    num_heads=first.heads if first else 1, num_kv_heads=first.kv_heads if first else 1, head_dim=first.dim if first else 64,
+    rms_norm_eps=float(cfg["norm"]["eps"]), rope_theta=getattr(first, "rot_base", 10000.0),
+    max_position_embeddings=int(cfg.get("max_positions", 1 << 20)), bos_token_id=int(cfg.get("bos_token_id", 0)),
+    eos_token_ids=tuple(cfg.get("eos_token_ids", ())), layer_specs=tuple(specs), block="sandwich", loop=loop,
+    norm_kind="layer", residual_mult=float(cfg.get("residual_mult", 1.0)), loop_input="add")
+
+
 def from_hf_config(cfg: dict) -> ModelConfig:
+  if cfg.get("architecture") == "Kopalorn":
+    return _kopalorn_config(cfg)
   if cfg.get("architecture") == "Nenizen":
     return _nenizen_config(cfg)
   if cfg.get("architecture") == "Tarepel":
@@ -847,6 +984,25 @@ TINY_NENIZEN = {
                "rot": {"base": 10000.0, "dims": 16}, "scale": 0.2}},
   ]}
 PRESETS["tiny-nenizen"] = _nenizen_config(TINY_NENIZEN)
+_TINY_GMOE = {"kind": "moe", "expert": {"ff": 40}, "shared": {"ff": 56},
+              "router": {"experts": 6, "top": 3, "scale": 1.5, "groups": {"count": 3, "keep": 2}}}
+TINY_KOPALORN = {
+  "architecture": "Kopalorn", "vocab": 304, "width": 112, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+  "loop": {"start": 1, "stop": 3, "times": 3},
+  "layers": [
+    {"type": "mlstm", "mlp": _TINY_GMOE, "mixer": {"heads": 2, "dim": 24, "vdim": 40, "gate_cap": 10.0}},
+    {"type": "attention", "mlp": _TINY_GMOE,
+     "mixer": {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 24, "diff": 0.3, "scale": 0.3, "mask": {"size": 21},
+               "rot": {"base": 10000.0, "dims": 8}}},
+    {"type": "parallel", "mlp": None,
+     "mixer": {"left": {"heads": 4, "kv_heads": 1, "dim": 24, "vdim": 16, "scale": 0.2},
+               "right": {"heads": 3, "dim": 16, "vdim": 24, "decay": [0.5, 0.9, 0.99]}}},
+    {"type": "attention", "mlp": {"kind": "moe", "expert": {"ff": 48}, "shared": None,
+                                  "router": {"experts": 4, "top": 1, "scale": 1.0, "groups": {"count": 1, "keep": 1}}},
+     "mixer": {"heads": 2, "kv_heads": 2, "dim": 32, "vdim": 32, "diff": 0.6, "scale": 0.18, "mask": {"size": 70},
+               "rot": {"base": 1000.0, "dims": 32}}},
+  ]}
+PRESETS["tiny-kopalorn"] = _kopalorn_config(TINY_KOPALORN)
 # aliases of the reference's model cards that share an architecture
 for _alias, _base in {"llama-3.1-70b-bf16": "llama-3.1-70b", "nemotron-70b": "llama-3.1-70b",
                       "deepseek-r1-distill-llama-70b": "llama-3.1-70b", "deepseek-r1-distill-llama-8b": "llama-3.1-8b",

@@ -102,8 +102,9 @@ class KVCache:
       dims = [c.layer_specs[i].kv_dims for i in ids]
       self.k = [None if a is None else torch.zeros(num_pages, a[0], PAGE, a[1], device=device, dtype=dtype) for a in dims]
       # (latent attention keeps no value pool: the cached latent is key and value, value dim 0)
-      self.v = [None if a is None or not a[2] else torch.zeros(num_pages, a[0], a[2], PAGE, device=device, dtype=dtype)
-                for a in dims]
+      # (key heads that share values: a fourth entry gives the value heads)
+      self.v = [None if a is None or not a[2] else
+                torch.zeros(num_pages, a[3] if len(a) > 3 else a[0], a[2], PAGE, device=device, dtype=dtype) for a in dims]
       # window attention with pooled blocks: per layer the (source layer, block size) pooled caches it reads, K
       # [pages, G, per, d] and V [pages, G, per, dv]; entries live with the page of a block's last token, so they are
       # handed out and returned with the sequence's pages.  pool_owner[j]: this layer fills them (the first layer of
@@ -145,7 +146,7 @@ class KVCache:
       for i in ids:
         a, w = c.layer_specs[i].kv_dims, c.layer_specs[i].wattn
         if a is not None:
-          n += a[0] * PAGE * (a[1] + a[2]) * itemsize
+          n += PAGE * (a[0] * a[1] + (a[3] if len(a) > 3 else a[0]) * a[2]) * itemsize
         if w is not None and w.pool > 0 and w.window > 0 and (w.kv_from if w.kv_from >= 0 else i, w.pool) not in seen:
           seen.add((w.kv_from if w.kv_from >= 0 else i, w.pool))
           n += w.kv_heads * K.pool_dims(w.pool) * (w.dim + w.vdim) * itemsize
@@ -167,25 +168,28 @@ class KVCache:
 class StatePool:
   """Recurrent state of a shard's layers, one slot per live request (models.config.LinearRecurrenceSpec): per layer
   with a recurrence S^T [slots, H, dv, d] fp32 (a value channel's key rows contiguous) and, for rules with short convolutions, the last taps - 1 convolution
-  inputs [slots, taps - 1, channels] fp32.  A slot is cleared when a request is admitted to it."""
+  inputs [slots, taps - 1, channels] fp32; rules that carry scalars per head beside the matrix (the mlstm's running maximum)
+  keep them in aux [slots, H, n] fp32.  A slot is cleared when a request is admitted to it."""
 
   def __init__(self, c: ModelConfig, layer_ids, slots: int, device):
     self.slots = slots
     self.S: List[Optional[torch.Tensor]] = []
     self.conv: List[Optional[torch.Tensor]] = []
+    self.aux: List[Optional[torch.Tensor]] = []
     for i, _ in c.layer_runs(layer_ids):  # (a looped layer: a state of its own in every pass)
-      sd = c.layer_specs[i].state_dims  # (heads, value dim, key dim, taps, convolution channels)
+      sd = c.layer_specs[i].state_dims  # (heads, value channels, key dim, taps, convolution channels, scalars per head)
       self.S.append(None if sd is None else torch.zeros(slots, sd[0], sd[1], sd[2], device=device, dtype=torch.float32))
       self.conv.append(torch.zeros(slots, max(sd[3] - 1, 0), sd[4], device=device, dtype=torch.float32)
                        if sd is not None and sd[4] else None)
+      self.aux.append(torch.zeros(slots, sd[0], sd[5], device=device, dtype=torch.float32) if sd is not None and sd[5] else None)
 
   def clear(self, slot: int) -> None:
-    for t in self.S + self.conv:
+    for t in self.S + self.conv + self.aux:
       if t is not None:
         t[slot].zero_()
 
   def nbytes(self) -> int:
-    return sum(t.numel() * 4 for t in self.S + self.conv if t is not None)
+    return sum(t.numel() * 4 for t in self.S + self.conv + self.aux if t is not None)
 
 
 class ShardModel:
@@ -215,7 +219,7 @@ class ShardModel:
                                       high_freq_factor=a.rot_scaling[2], original_max_position_embeddings=a.rot_scaling[3])
           self.rope_tabs[(a.rot_dims, a.rot_base, a.rot_scaling)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base,
                                                                                  sc, self.device)
-        a = c.layer_specs[i].lattn
+        a = c.layer_specs[i].lattn or c.layer_specs[i].dattn
         if a is not None and a.rot_dims and (a.rot_dims, a.rot_base) not in self.rope_tabs:
           self.rope_tabs[(a.rot_dims, a.rot_base)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base, None, self.device)
       self.runs = c.layer_runs(self.layer_ids)
@@ -548,8 +552,57 @@ class ShardModel:
       K.kv_pool_update(self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q, inp.ctx_lens,
                        a.pool, inp.max_qlen)
     pool = a.pool if self.kv.kp[j] is not None else 0
+    n = a.heads * a.vdim
+    o = mix[:, :n] if a.gate == "none" else torch.empty(P.shape[0], n, dtype=torch.float32, device=P.device)
     K.attn_window_pool(q, self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q,
-                       inp.ctx_lens, lw.sink, a.scale, a.window, pool, mix[:, :a.heads * a.vdim], max_qlen=inp.max_qlen)
+                       inp.ctx_lens, lw.sink, a.scale, a.window, pool, o, max_qlen=inp.max_qlen)
+    if a.gate != "none":  # one sigmoid gate per element, from the mixer's input
+      K.sigmoid_gate_mul(o, P, lw.cols["gate"][0], mix)
+
+  def _diff_attn(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Differential attention on the window-attention kernels: the two maps of every head are query heads of their own
+    (the fused projection orders them kv head, map, head of the group) over 2 G key heads that share G value heads;
+    then a_1 - lam a_2, the per-head RMS division and the per-head gate."""
+    a = lw.spec.dattn
+    T, dev = P.shape[0], P.device
+    q = torch.empty(T, 2 * a.heads, a.dim, dtype=mix.dtype, device=dev)
+    tab = self.rope_tabs.get((a.rot_dims, a.rot_base))
+    K.qk_norm_rope_store(P, None, lw.cols["q"][0], lw.cols["k"][0], lw.cols["v"][0], 2 * a.heads, 2 * a.kv_heads, a.dim, a.vdim,
+                         a.rot_dims if tab is not None else 0, inp.positions,
+                         tab if tab is not None else torch.zeros(1, 0, device=dev), inp.slots, self.c.rms_norm_eps, False, q,
+                         self.kv.k[j], self.kv.v[j])
+    o = torch.empty(T, 2 * a.heads * a.vdim, dtype=torch.float32, device=dev)
+    K.attn_window_pool(q, self.kv.k[j], self.kv.v[j], None, None, inp.block_tables, inp.cu_q, inp.ctx_lens, None, a.scale,
+                       a.window, 0, o, max_qlen=inp.max_qlen)
+    K.diff_attn_out(o, P, lw.cols["gate"][0], a.heads, a.kv_heads, lw.lam, 1.0 - a.lam_init, self.c.rms_norm_eps, mix)
+
+  def _mlstm(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """The xLSTM matrix memory on the state slots: gates and the running maximum per head, the framework's linear
+    recurrence with one decay per head and an input scale (the normaliser is the state's last value channel), then the
+    stabilised division, the per-head norm, the weight and the sigmoid gate."""
+    r, st, dev = lw.spec.rec, self.state, P.device
+    T, H = P.shape[0], r.heads
+    decay, inscale, m = (torch.empty(T, H, dtype=torch.float32, device=dev) for _ in range(3))
+    K.mlstm_gates(P, lw.cols["ri"][0], lw.cols["rf"][0], lw.gate_b, r.gate_cap, st.aux[j].view(-1, H), inp.state_slots, inp.cu_q, decay,
+                  inscale, m)
+    o = torch.empty(T, H * (r.vdim + 1), dtype=torch.float32, device=dev)
+    (qo, qn), (ko, kn), (vo, vn) = lw.cols["rq"], lw.cols["rk"], lw.cols["rv"]
+    K.linear_recurrence(P[:, qo:qo + qn], P[:, ko:ko + kn], P[:, vo:vo + vn], decay, inscale, r.dim ** -0.5, st.S[j],
+                        inp.state_slots, inp.cu_q, o)
+    K.gated_group_norm(o, m, lw.rec_norm, P, lw.cols["rg"][0], H, self.c.rms_norm_eps, mix)
+
+  def _lightning(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Lightning attention on the state slots: SiLU on q, k, v, the linear recurrence with one fixed decay per head, the
+    norm over all heads together, the weight and the sigmoid gate."""
+    r, st, dev = lw.spec.rec, self.state, P.device
+    T, H = P.shape[0], r.heads
+    nq, nv = H * r.dim, H * r.vdim
+    qkv = torch.empty(T, 2 * nq + nv, dtype=torch.float32, device=dev)
+    K.silu_cols(P, lw.cols["rq"][0], 2 * nq + nv, qkv)  # (q | k | v are neighbours in the fused projection)
+    o = torch.empty(T, nv, dtype=torch.float32, device=dev)
+    K.linear_recurrence(qkv[:, :nq], qkv[:, nq:2 * nq], qkv[:, 2 * nq:], lw.decay.expand(T, H).contiguous(), None, 1.0,
+                        st.S[j], inp.state_slots, inp.cu_q, o)
+    K.gated_group_norm(o, None, lw.rec_norm, P, lw.cols["rg"][0], 1, self.c.rms_norm_eps, mix)
 
   def _ssd(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
     """Mamba-2 mixer on the state slots: convolution + SiLU, step sizes and decays, the recurrence on the fp32 state
@@ -569,24 +622,33 @@ class ShardModel:
     K.ssd_gate_norm(o, xbc, lw.skip_d, P, i0, lw.ssd_norm, m.norm_groups, self.c.rms_norm_eps, mix)
 
   def _relu2_moe(self, hn: torch.Tensor, P: torch.Tensor, lw, rows) -> torch.Tensor:
-    """Routed relu^2 experts + the gated shared expert -> fp32 [T, D].  Routing on the framework's top-k kernel (the
-    softmax over the chosen logits), experts on the grouped GEMMs (bf16) or per expert on the vendor SGEMM (fp32)."""
+    """Routed relu^2 experts + the gated shared expert -> fp32 [T, D].  Routing on the framework's top-k kernels (the
+    softmax over the chosen logits, or the grouped sigmoid rule with a correction), experts on the grouped GEMMs (bf16)
+    or per expert on the vendor SGEMM (fp32)."""
     f, dev = lw.spec.ffn, P.device
     T, D = hn.shape[0], self.c.hidden_size
     E, k = f.experts, f.top
     r0 = lw.ff_cols["router"][0]
-    logits = (P[:, r0:r0 + E] + lw.router_b).contiguous()
+    grouped = f.route == "sigmoid_groups"  # sigmoid scores, choice among the best groups on the corrected scores
+    logits = P[:, r0:r0 + E].contiguous() if grouped else (P[:, r0:r0 + E] + lw.router_b).contiguous()
     if P.is_cuda:
       topw = torch.empty(T * k, dtype=torch.float32, device=dev)
       topi, slot_of, sorted_tok = (torch.empty(T * k, dtype=torch.int32, device=dev) for _ in range(3))
       off = torch.empty(E + 1, dtype=torch.int32, device=dev)
-      if E <= 64 and k <= 8:
+      if grouped:
+        K.moe_route_ds(logits, lw.router_b, k, f.groups, f.keep, 2, True, True, f.route_scale,
+                       outs=(topw, topi, slot_of, sorted_tok, off))
+      elif E <= 64 and k <= 8:
         require().moe_route(logits, k, topw, topi, slot_of, sorted_tok, off)
       else:
         K.moe_route_ds(logits, None, k, 1, 1, 0, False, True, 1.0, outs=(topw, topi, slot_of, sorted_tok, off))
     else:
-      val, idx = torch.topk(logits, k, dim=-1)
-      topw, topi = torch.softmax(val, -1).reshape(-1), idx.reshape(-1).int()
+      if grouped:
+        topw, idx = K.moe_route_ds(logits, lw.router_b, k, f.groups, f.keep, 2, True, True, f.route_scale)
+        topw, topi = topw.reshape(-1), idx.reshape(-1).int()
+      else:
+        val, idx = torch.topk(logits, k, dim=-1)
+        topw, topi = torch.softmax(val, -1).reshape(-1), idx.reshape(-1).int()
       order = torch.argsort(topi, stable=True)
       slot_of = torch.empty_like(order)
       slot_of[order] = torch.arange(T * k)
@@ -768,13 +830,17 @@ class ShardModel:
     return out
 
   def _forward_sandwich(self, h: torch.Tensor, inp: StepInputs, adt) -> torch.Tensor:
-    """Layer runs (a looped layer once per pass, each pass with caches of its own) of sandwich blocks on the fp32
-    stream h (hn: the normed sublayer input in the GEMMs' operand dtype):
-      pass start:  h <- [h | embedding output] @ loop_in^T + step[pass]
-      P = hn @ in_w^T                    queries (or their latent), kv latent, rotated key part, output gate
-      h += norm1b(latent_attention(P) @ out_w^T);  hn = norm2(h)
-      P = hn @ ff_w^T                    gate | up, or router | shared gate | shared up
-      h += norm2b(ff(P));  hn = the next run's norm1(h)
+    """Layer runs (a looped layer once per pass, each pass with caches and states of its own) of sandwich blocks on the
+    fp32 stream h (hn: the normed sublayer input in the GEMMs' operand dtype):
+      pass start:  h <- [h | embedding output] @ loop_in^T + step[pass]       (loop_input "linear")
+                   h <- h + embedding output (passes after the first) + step[pass]       ("add")
+      P = hn @ in_w^T                    every projection that reads the mixer's input
+      h += mult * norm1b(mixer(P) @ out_w^T);  hn = norm2(h)
+      P = hn @ ff_w^T                    gate | up, or router | shared expert's projections
+      h += mult * norm2b(ff(P));  hn = the next run's norm1(h)
+    The norms are RMS norms with a weight, or (norm_kind "layer") layer norms with weight and bias.  Mixers: latent
+    attention; differential attention; mlstm; gated attention beside lightning attention, each projected to the width,
+    RMS-normed with its own weight and averaged.
     Returns h (non-last shard) or softcap(head(final_norm(h rows inp.last_idx)))."""
     c, w = self.c, self.w
     T, D = h.shape
@@ -791,43 +857,66 @@ class ShardModel:
     if w.loop_in is not None:  # the embedding output in the operand dtype, second half of every pass's input rows
       xx = torch.zeros(T, 2 * Dp, dtype=adt, device=h.device)
       xx[:, Dp:Dp + D] = h.to(adt)
+    elif w.loop_step is not None:
+      x0 = h.clone()
     runs = self.runs
-    eps = c.rms_norm_eps
+    eps, mult = c.rms_norm_eps, c.residual_mult
     fresh = True  # hn does not hold this run's normed input yet
     for j, (li, t) in enumerate(runs):
       lw = w.layers[li]
       s = lw.spec
-      if t >= 0:
+      if t >= 0 and w.loop_in is not None:
         xx[:, :D] = h.to(adt)
         h = self._proj(xx, w.loop_in)[:, :D] + w.loop_step[t]
         fresh = True
+      elif t >= 0:
+        if t > 0:
+          h += x0
+        h += w.loop_step[t]
+        fresh = True
       if fresh:
-        K.sandwich_add_norm(h, None, None, lw.norm1, eps, hn)
+        K.sandwich_add_norm(h, None, None, lw.norm1, eps, hn, bn=lw.norm1_b)
       P = self._proj(hn, lw.in_w)
       mix = rows("mix", lw.mix_cols["mix"][1], lw.out_w.shape[1])
-      self._latent_attn(P, lw, j, inp, mix, rows)
+      if s.lattn is not None:
+        self._latent_attn(P, lw, j, inp, mix, rows)
+      elif s.dattn is not None:
+        self._diff_attn(P, lw, j, inp, mix)
+      elif s.wattn is not None:
+        self._window_attn(P, lw, j, inp, mix)
+      else:
+        self._mlstm(P, lw, j, inp, mix)
       y = self._proj(mix, lw.out_w)
+      if s.wattn is not None and s.rec is not None:  # the second mixer of a parallel layer, then the mean of the normed pair
+        mix2 = rows("mix2", lw.mix_cols["mix2"][1], lw.out2_w.shape[1])
+        self._lightning(P, lw, j, inp, mix2)
+        y2 = self._proj(mix2, lw.out2_w)
+        y1, y = y, torch.empty(T, D, dtype=torch.float32, device=h.device)
+        K.pair_norm_mean(y1, y2, lw.pair_w, eps, y)
       f = s.ffn
       # the norm that follows this run: the next run's input norm unless a pass starts there
-      nxt = w.layers[runs[j + 1][0]].norm1 if j + 1 < len(runs) and runs[j + 1][1] < 0 else None
+      nl = w.layers[runs[j + 1][0]] if j + 1 < len(runs) and runs[j + 1][1] < 0 else None
+      nxt, nxt_b = (nl.norm1, nl.norm1_b) if nl is not None else (None, None)
       if f is None:
-        K.sandwich_add_norm(h, y, lw.norm1b, nxt, eps, hn)
+        K.sandwich_add_norm(h, y, lw.norm1b, nxt, eps, hn, bb=lw.norm1b_b, bn=nxt_b, mult=mult)
       else:
-        K.sandwich_add_norm(h, y, lw.norm1b, lw.norm2, eps, hn)
+        K.sandwich_add_norm(h, y, lw.norm1b, lw.norm2, eps, hn, bb=lw.norm1b_b, bn=lw.norm2_b, mult=mult)
         P = self._proj(hn, lw.ff_w)
         if f.kind == "clamped_glu":
           act = rows("act", f.ff, lw.down_w.shape[1])
           K.glu_act(P, lw.ff_cols["gate"][0], lw.ff_cols["up"][0], f.ff, True, f.limit, act)
           y = self._proj(act, lw.down_w)
+        elif f.kind == "relu2_moe":
+          y = self._relu2_moe(hn, P, lw, rows)
         else:
           y = self._silu_moe(hn, P, lw, rows)
-        K.sandwich_add_norm(h, y, lw.norm2b, nxt, eps, hn)
+        K.sandwich_add_norm(h, y, lw.norm2b, nxt, eps, hn, bb=lw.norm2b_b, bn=nxt_b, mult=mult)
       fresh = nxt is None
     if not self.shard.is_last_layer():
       return h
     hl = h.index_select(0, inp.last_idx)
     xn = torch.zeros(hl.shape[0], Dp, dtype=adt, device=h.device)
-    K.sandwich_add_norm(hl, None, None, w.norm, eps, xn)
+    K.sandwich_add_norm(hl, None, None, w.norm, eps, xn, bn=w.norm_b)
     logits = self._proj(xn, w.lm_head)[:, :c.vocab_size]
     if c.logit_softcap > 0:
       logits = torch.tanh(logits / c.logit_softcap) * c.logit_softcap

@@ -75,6 +75,7 @@ class ShardWeights:
   layers: Dict[int, LayerWeights] = field(default_factory=dict)
   embed: Optional[torch.Tensor] = None  # first shard (and last, when tied)
   norm: Optional[torch.Tensor] = None  # last shard
+  norm_b: Optional[torch.Tensor] = None  # last shard, models whose norms are layer norms with a bias
   lm_head: Optional[torch.Tensor] = None  # last shard (aliases embed when tied)
   vision: Optional[Dict[str, torch.Tensor]] = None  # LLaVA tower + projector (first shard), HF names
   # looped layers (config.loop): the pass input mix [Dn, 2 D padded] over [x | embedding output] and the vector added
@@ -93,7 +94,7 @@ class ShardWeights:
   def all_tensors(self) -> Iterable[torch.Tensor]:
     for lw in self.layers.values():
       yield from lw.tensors().values()
-    for t in (self.embed, self.norm, self.lm_head, self.loop_in, self.loop_step):
+    for t in (self.embed, self.norm, self.norm_b, self.lm_head, self.loop_in, self.loop_step):
       if t is not None:
         yield t
     if self.vision:
@@ -343,7 +344,7 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
     for lw in sw.layers.values():
       if lw.in_w.dtype == torch.bfloat16:
         lw.in_w, lw.out_w, lw.down_w, lw.ff_w = wide(lw.in_w), wide(lw.out_w), wide(lw.down_w), wide(lw.ff_w)
-        lw.uq_w = wide(lw.uq_w)
+        lw.uq_w, lw.out2_w = wide(lw.uq_w), wide(lw.out2_w)
         lw.ex_up_w, lw.ex_down_w = conv(lw.ex_up_w), conv(lw.ex_down_w)  # experts: shuffled per expert
     if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
       sw.lm_head = wide(sw.lm_head)
@@ -732,6 +733,20 @@ class MixedLayerWeights:
   uq_w: Optional[torch.Tensor] = None  # [H (dim + rot_dim) padded, q_rank padded]
   uk_w: Optional[torch.Tensor] = None  # [H, dim, kv_rank]: q_lat = q_unrotated . W_uk per head
   uv_w: Optional[torch.Tensor] = None  # [H, kv_rank, vdim]: o = o_lat . W_uv^T per head (stored transposed)
+  # sandwich blocks with layer norms: the four norms' biases; differential attention: `in_w` = [q (heads regrouped as
+  # kv head, map, head of the group; rotary dims in pair order) | k | v | one gate per head], lam = the layer's
+  # lambda; mlstm: [q | k | v | output gate | input gate | forget gate] and gate_b = [i bias | f bias]; a parallel layer:
+  # [attention q | k | v | gate | lightning q | k | v | gate], two output projections (out_w: attention, out2_w:
+  # lightning) and pair_w [2, D] = the weights of the norms over their results; decay [H] = lightning's decays
+  norm1_b: Optional[torch.Tensor] = None  # [D] fp32
+  norm1b_b: Optional[torch.Tensor] = None
+  norm2_b: Optional[torch.Tensor] = None
+  norm2b_b: Optional[torch.Tensor] = None
+  out2_w: Optional[torch.Tensor] = None
+  pair_w: Optional[torch.Tensor] = None
+  decay: Optional[torch.Tensor] = None
+  gate_b: Optional[torch.Tensor] = None
+  lam: float = 0.0
 
   def tensors(self) -> Dict[str, torch.Tensor]:
     return {k: v for k, v in self.__dict__.items() if isinstance(v, torch.Tensor)}
@@ -914,6 +929,124 @@ def build_sandwich_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayer
   return lw
 
 
+def _pair_order(d: int, R: int) -> torch.Tensor:
+  """Row order of one head whose rotation pairs (2i, 2i + 1) become (i, i + R / 2), the kernels' layout: a
+  permutation of the head's dims, applied to queries and keys alike, leaves every score as it was."""
+  return torch.tensor(list(range(0, R, 2)) + list(range(1, R, 2)) + list(range(R, d)), dtype=torch.long)
+
+
+def _relu2_moe_weights(lw: MixedLayerWeights, f, get, q: str, D: int, dev, dtype, gate_rows=None):
+  """Router | shared up | shared gate (| the sublayer's gate) fused into ff_w, experts stacked and padded."""
+  fb = [("router", get(q + "router"))]
+  down = None
+  if f.shared_ff:
+    fb += [("sh_up", get(q + "shared.up")), ("sh_gate", get(q + "shared.sg").reshape(1, D))]
+    down = get(q + "shared.down")
+  Fp, Dp = _up(f.ff, 128), _up(D, 128)
+  lw.ex_up_w = dev(torch.stack([_pad2(get(q + f"e{e}.up"), Fp, Dp) for e in range(f.experts)]), dtype)
+  lw.ex_down_w = dev(torch.stack([_pad2(get(q + f"e{e}.down"), Dp, Fp) for e in range(f.experts)]), dtype)
+  if gate_rows is not None:
+    fb.append(("gate", gate_rows))
+  ff_w, lw.ff_cols = _fused_rows(fb, D)
+  lw.ff_w = dev(ff_w, dtype)
+  if down is not None:
+    lw.down_w = dev(_pad2(down, _up(D, 64), _up(down.shape[1], 128)), dtype)
+
+
+def build_ln_sandwich_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWeights:
+  """One layer-norm sandwich layer (differential attention, mlstm, or gated attention beside lightning attention;
+  relu^2 experts with grouped sigmoid routing) from `get(name)`."""
+  def dev(t, dt=torch.float32):
+    return t.to(device=device, dtype=dt).contiguous()
+  m = p + "mix."
+  a, w, r, f = spec.dattn, spec.wattn, spec.rec, spec.ffn
+  bias, out2 = {}, None
+  if a is not None:
+    rep, d = a.heads // a.kv_heads, a.dim
+    order = _pair_order(d, a.rot_dims)
+    q = get(m + "q").reshape(a.kv_heads, rep, 2, d, D).permute(0, 2, 1, 3, 4)[:, :, :, order]  # [kv head, map, head, d]
+    k = get(m + "k").reshape(a.kv_heads, 2, d, D)[:, :, order]
+    blocks = [("q", q.reshape(-1, D)), ("k", k.reshape(-1, D)), ("v", get(m + "v")), ("gate", get(m + "g"))]
+    out = get(m + "o")
+  elif w is not None:
+    l, rr = m + "left.", m + "right."
+    blocks = [(n, get(l + n)) for n in ("q", "k", "v")] + [("gate", get(l + "g"))]
+    bias = {n: get(l + n + ".b") for n in ("q", "k", "v")}
+    blocks += [("rq", get(rr + "q")), ("rk", get(rr + "k")), ("rv", get(rr + "v")), ("rg", get(rr + "g"))]
+    out, out2 = get(l + "o"), get(rr + "o")
+  else:
+    blocks = [("rq", get(m + "q")), ("rk", get(m + "k")), ("rv", get(m + "v")), ("rg", get(m + "g")), ("ri", get(m + "i")),
+              ("rf", get(m + "f"))]
+    out = get(m + "o")
+  in_w, cols = _fused_rows(blocks, D)
+  lw = MixedLayerWeights(spec, dev(in_w, dtype), cols, dev(_pad2(out, _up(D, 64), _up(out.shape[1], 128)), dtype),
+                         {"mix": (0, out.shape[1])})
+  for n in ("norm1", "norm1b") + (("norm2", "norm2b") if f is not None else ()):
+    setattr(lw, n, dev(get(p + n)))
+    setattr(lw, n + "_b", dev(get(p + n + ".b")))
+  if a is not None:
+    lam = torch.exp((get(m + "lq1") * get(m + "lk1")).sum()) - torch.exp((get(m + "lq2") * get(m + "lk2")).sum()) + a.lam_init
+    lw.lam = float(lam)
+  if bias:
+    b = torch.zeros(in_w.shape[0])
+    for n, t in bias.items():
+      b[cols[n][0]:cols[n][0] + cols[n][1]] = t
+    lw.in_b = dev(b)
+  if out2 is not None:
+    lw.out2_w = dev(_pad2(out2, _up(D, 64), _up(out2.shape[1], 128)), dtype)
+    lw.mix_cols["mix2"] = (0, out2.shape[1])
+    lw.pair_w = dev(torch.stack([get(m + "left.out"), get(m + "right.out")]))
+    lw.rec_norm = dev(get(m + "right.norm"))
+    lw.decay = dev(torch.tensor(r.decays))
+  elif r is not None:
+    lw.rec_norm = dev(get(m + "norm"))
+    lw.gate_b = dev(torch.cat([get(m + "i.b"), get(m + "f.b")]))
+  if f is not None:
+    _relu2_moe_weights(lw, f, get, p + "mlp.", D, dev, dtype)
+    lw.router_b = dev(get(p + "mlp.correction"))
+  return lw
+
+
+def ln_sandwich_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
+  """Name -> shape of every tensor of a layer-norm sandwich checkpoint (Kopalorn)."""
+  D, out = c.hidden_size, {}
+  out["embed"] = (c.vocab_size, D)
+  if c.loop:
+    out["loop.step"] = (c.loop[2], D)
+  for i, s in enumerate(c.layer_specs):
+    p, m = f"l{i}.", f"l{i}.mix."
+    a, w, r, f = s.dattn, s.wattn, s.rec, s.ffn
+    for n in ("norm1", "norm1b") + (("norm2", "norm2b") if f is not None else ()):
+      out[p + n], out[p + n + ".b"] = (D,), (D,)
+    if a is not None:
+      out[m + "q"], out[m + "k"], out[m + "v"] = (2 * a.heads * a.dim, D), (2 * a.kv_heads * a.dim, D), (a.kv_heads * a.vdim, D)
+      for n in ("lq1", "lk1", "lq2", "lk2"):
+        out[m + n] = (a.dim,)
+      out[m + "g"], out[m + "o"] = (a.heads, D), (D, a.heads * a.vdim)
+    elif w is not None:
+      l, rr = m + "left.", m + "right."
+      for n, rows in (("q", w.heads * w.dim), ("k", w.kv_heads * w.dim), ("v", w.kv_heads * w.vdim)):
+        out[l + n], out[l + n + ".b"] = (rows, D), (rows,)
+      out[l + "g"], out[l + "o"] = (w.heads * w.vdim, D), (D, w.heads * w.vdim)
+      out[rr + "q"], out[rr + "k"], out[rr + "v"] = (r.heads * r.dim, D), (r.heads * r.dim, D), (r.heads * r.vdim, D)
+      out[rr + "g"], out[rr + "o"], out[rr + "norm"] = (r.heads * r.vdim, D), (D, r.heads * r.vdim), (r.heads * r.vdim,)
+      out[l + "out"], out[rr + "out"] = (D,), (D,)
+    else:
+      out[m + "q"], out[m + "k"], out[m + "v"] = (r.heads * r.dim, D), (r.heads * r.dim, D), (r.heads * r.vdim, D)
+      out[m + "g"], out[m + "o"], out[m + "norm"] = (r.heads * r.vdim, D), (D, r.heads * r.vdim), (r.heads * r.vdim,)
+      out[m + "i"], out[m + "i.b"], out[m + "f"], out[m + "f.b"] = (r.heads, D), (r.heads,), (r.heads, D), (r.heads,)
+    if f is None:
+      continue
+    q = p + "mlp."
+    for e in range(f.experts):
+      out[q + f"e{e}.up"], out[q + f"e{e}.down"] = (f.ff, D), (D, f.ff)
+    out[q + "router"], out[q + "correction"] = (f.experts, D), (f.experts,)
+    if f.shared_ff:
+      out[q + "shared.up"], out[q + "shared.down"], out[q + "shared.sg"] = (f.shared_ff, D), (D, f.shared_ff), (1, D)
+  out["final.norm"], out["final.norm.b"], out["head"] = (D,), (D,), (c.vocab_size, D)
+  return out
+
+
 def sandwich_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
   """Name -> shape of every tensor of a sandwich-block checkpoint (Nenizen); the LM head is the embedding table."""
   D, out = c.hidden_size, {}
@@ -995,7 +1128,7 @@ def mixed_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
   if c.block == "postln":
     return postln_tensor_shapes(c)
   if c.block == "sandwich":
-    return sandwich_tensor_shapes(c)
+    return ln_sandwich_tensor_shapes(c) if c.norm_kind == "layer" else sandwich_tensor_shapes(c)
   D, out = c.hidden_size, {}
   out["embed"] = (c.vocab_size, D)
   for i, s in enumerate(c.layer_specs):
@@ -1032,6 +1165,15 @@ def random_mixed_tensors(c: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
     leaf = name.split(".")[-1]
     if name.endswith(".conv"):
       t = torch.randn(shape, generator=g) * 0.5
+    elif c.norm_kind == "layer" and leaf in ("b", "correction", "out", "lq1", "lk1", "lq2", "lk2"):
+      # norm biases, projection biases, gate biases (forget gates mostly open), the router's correction (large enough to
+      # change the choice), the lambda vectors
+      kind = name.split(".")[-2]
+      t = {"b": torch.randn(shape, generator=g) * (0.1 if kind.startswith("norm") else 0.5) + (2.0 if kind == "f" else 0.0),
+           "correction": torch.randn(shape, generator=g) * 0.3,
+           "out": 1.0 + 0.1 * torch.randn(shape, generator=g)}.get(leaf)
+      if t is None:
+        t = torch.randn(shape, generator=g) * 0.4
     elif leaf in ("sink", "D", "act") or (leaf == "b" and c.block == "postln"):
       t = torch.randn(shape, generator=g) * (0.5 if leaf == "b" else 1.0)
     elif leaf in ("norm1", "norm2", "norm1b", "norm2b") or name == "final.norm":
@@ -1061,12 +1203,16 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
   sw = ShardWeights(c, shard)
   D = c.hidden_size
   build = {"postln": build_postln_layer, "sandwich": build_sandwich_layer}.get(c.block, build_mixed_layer)
+  if c.block == "sandwich" and c.norm_kind == "layer":
+    build = build_ln_sandwich_layer
   for i in shard.layers():
     sw.layers[i] = build(c.layer_specs[i], get, f"l{i}.", D, device, dtype)
   if shard.is_first_layer():
     # gathered into the fp32 residual; a model that scales its embedding output gathers from the scaled table
     sw.embed = (get("embed") * c.embed_scale).to(device=device, dtype=torch.float32).contiguous()
-  if c.loop and any(c.loop[0] <= i < c.loop[1] for i in shard.layers()):
+  if c.loop and c.loop_input == "add" and any(c.loop[0] <= i < c.loop[1] for i in shard.layers()):
+    sw.loop_step = get("loop.step").to(device=device, dtype=torch.float32).contiguous()
+  elif c.loop and any(c.loop[0] <= i < c.loop[1] for i in shard.layers()):
     w_in = get("loop.in")  # [D, 2 D] over [x | embedding output]: each half padded to the GEMM's K tile
     Dp = _up(D, 128)
     li = torch.zeros(_up(D, 64), 2 * Dp)
@@ -1075,6 +1221,8 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
     sw.loop_step = get("loop.step").to(device=device, dtype=torch.float32).contiguous()
   if shard.is_last_layer():
     sw.norm = get("final.norm").reshape(-1).to(device=device, dtype=torch.float32)
+    if c.norm_kind == "layer":
+      sw.norm_b = get("final.norm.b").reshape(-1).to(device=device, dtype=torch.float32)
     head = torch.zeros(_up(c.vocab_size, 64), _up(D, 128))
     head[:c.vocab_size, :D] = get("embed" if c.tie_word_embeddings and c.is_mixed else "head")
     sw.lm_head = head.to(device=device, dtype=dtype).contiguous()

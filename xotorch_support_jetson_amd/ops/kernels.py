@@ -490,7 +490,9 @@ def gla_prep(P, a1_off: int, a2, a2_b, tau: float, decay) -> None:
 def linear_recurrence(q, k, v, decay, beta, q_scale: float, state, state_slots, cu_q, out) -> None:
   """Per sequence and value head, token by token on the fp32 state, stored S^T [slots, H, dv, d] (updated in place):
   beta given (delta rule, decay [T, H]):  S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q
-  else (decay [T, H d] per key channel):  S = diag(a) S + k v^T; o = S^T q.      q is scaled by q_scale."""
+  else (decay [T, H d] per key channel, or [T, H] per head):  S = diag(a) S + k v^T; o = S^T q.   q is scaled by q_scale.
+  A state with one value channel more than v has (decay [T, H], beta [T, H] an input scale): S = g S + k (beta [v | 1])^T,
+  the last channel being a normaliser n = g n + beta k; out [T, H (dv + 1)] then ends each head with n . q."""
   _mix("linear_recurrence", _gpu(q))(q, k, v, decay, beta, float(q_scale), state, state_slots, cu_q, out)
 
 
@@ -513,7 +515,8 @@ def qk_norm_rope_store(P, bias, q_off: int, k_off: int, v_off: int, H: int, G: i
                        slots, eps: float, qk_norm: bool, q_out, k_cache, v_cache) -> None:
   """q / k / v = P's columns (+ bias, one fp32 number per column of P); rotate-half RoPE on the first R dims of every
   q / k head, then (qk_norm) each head divided by its RMS; q -> q_out [T, H, d], k -> k_cache [pages, G, 64, d],
-  v -> v_cache [pages, G, dv, 64] at `slots`.  k_off < 0: the layer has no keys and values of its own."""
+  v -> v_cache [pages, Gv, dv, 64] at `slots` (Gv = v_cache's heads: G, or fewer when neighbouring key heads share a
+  value head).  k_off < 0: the layer has no keys and values of its own."""
   _mix("qk_norm_rope_store", _gpu(P))(P, bias, int(q_off), int(k_off), int(v_off), int(H), int(G), int(d), int(dv), int(R),
                                       pos, cos_sin, slots, float(eps), bool(qk_norm), q_out, k_cache, v_cache)
 
@@ -528,7 +531,8 @@ def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool:
 def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, scale: float, window: int,
                      pool: int, out, max_qlen: int = 0) -> None:
   """out [T, H dv] = softmax attention of each new token over the tokens at most window - 1 places back (window 0:
-  all), the pooled blocks that end at or before position - window (pool 0: none), and the per-head sink logit."""
+  all), the pooled blocks that end at or before position - window (pool 0: none), and the per-head sink logit.  Key
+  head g reads value head g / (G / Gv) (the caches' head counts); out may be fp32 beside bf16 caches."""
   _mix("attn_window_pool", _gpu(q))(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, float(scale),
                                     int(window), int(pool), out, int(max_qlen) or int(q.shape[0]))
 
@@ -564,10 +568,11 @@ def moe_weighted_sum(y, slot_of, topw, k: int, sh_y, P, shg_off: int, out, split
 
 
 # ------------------------------------------------------------------ sandwich blocks (csrc/latent.hip)
-def sandwich_add_norm(x, y, wb, wn, eps: float, out=None) -> None:
-  """fp32 stream rows x [T, D] += y / rms(y) * wb in place (y None: nothing is added); with wn, out[:, :D] =
-  x / rms(x) * wn in out's dtype (the next GEMM's operand)."""
-  _mix("sandwich_add_norm", _gpu(x))(x, y, wb, wn, float(eps), out)
+def sandwich_add_norm(x, y, wb, wn, eps: float, out=None, bb=None, bn=None, mult: float = 1.0) -> None:
+  """fp32 stream rows x [T, D] += mult * norm(y) * wb in place (y None: nothing is added); with wn, out[:, :D] =
+  norm(x) * wn in out's dtype (the next GEMM's operand).  norm = division by the RMS, or, with the biases bb / bn, the
+  layer norm (v - mean) / sqrt(var + eps) * w + b."""
+  _mix("sandwich_add_norm", _gpu(x))(x, y, wb, wn, float(eps), out, bb, bn, float(mult))
 
 
 def latent_kv_store(P, ckv_off: int, R: int, dr: int, kv_norm, q_off: int, q_rank: int, q_norm, eps: float, rot_dims: int,
@@ -608,3 +613,39 @@ def glu_act(P, gate_off: int, up_off: int, F: int, clamped: bool, limit: float, 
   """out[:, :F] = silu(g) * u, or (clamped) g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u,
   -limit, limit); g = P[:, gate_off : +F], u = P[:, up_off : +F]."""
   _mix("glu_act", _gpu(P))(P, int(gate_off), int(up_off), int(F), bool(clamped), float(limit), out)
+
+
+# ------------------------------------------------------------------ layer-norm sandwich blocks (csrc/recurrent_gates.hip)
+def diff_attn_out(a, P, g_off: int, H: int, G: int, lam: float, post: float, eps: float, out) -> None:
+  """Differential attention's combination: a [T, 2 H dv] fp32, the two maps' outputs with heads ordered (kv head, map, head
+  of the group) -> out[:, :H dv] = rms_norm(a_1 - lam a_2) * post * sigmoid(P[:, g_off + head])."""
+  _mix("diff_attn_out", _gpu(a))(a, P, int(g_off), int(H), int(G), float(lam), float(post), float(eps), out)
+
+
+def sigmoid_gate_mul(a, P, g_off: int, out) -> None:
+  """out[:, :n] = a * sigmoid(P[:, g_off : +n]) for a [T, n]."""
+  _mix("sigmoid_gate_mul", _gpu(a))(a, P, int(g_off), out)
+
+
+def silu_cols(P, off: int, n: int, out) -> None:
+  """out [T, n] fp32 = silu(P[:, off : +n])."""
+  _mix("silu_cols", _gpu(P))(P, int(off), int(n), out)
+
+
+def mlstm_gates(P, i_off: int, f_off: int, gate_b, cap: float, mstate, state_slots, cu_q, decay, inscale, mout) -> None:
+  """The mlstm's gates of a step, per head: i = cap tanh((P[i_off + h] + gate_b[h]) / cap), f = logsigmoid(cap tanh((P[f_off
+  + h] + gate_b[H + h]) / cap)), the running maximum m_t = max(f + m_(t-1), i) continued from mstate [slots, H] (updated
+  in place); decay [T, H] = e^(f + m_(t-1) - m_t), inscale = e^(i - m_t), mout = m_t."""
+  _mix("mlstm_gates", _gpu(P))(P, int(i_off), int(f_off), gate_b, float(cap), mstate, state_slots, cu_q, decay, inscale, mout)
+
+
+def gated_group_norm(o, m, w, P, g_off: int, groups: int, eps: float, out) -> None:
+  """out[:, :groups gs] = o's values divided by their group's RMS, times w, times sigmoid(P[:, g_off : ...]).  With m
+  [T, groups] every group of o carries one channel more, a normaliser n, and its values are first divided by max(|n|,
+  e^(-m)) + 1e-6."""
+  _mix("gated_group_norm", _gpu(o))(o, m, w, P, int(g_off), int(groups), float(eps), out)
+
+
+def pair_norm_mean(y1, y2, w, eps: float, out) -> None:
+  """out [T, D] fp32 = (rms_norm(y1) * w[0] + rms_norm(y2) * w[1]) / 2."""
+  _mix("pair_norm_mean", _gpu(y1))(y1, y2, w, float(eps), out)

@@ -220,7 +220,7 @@ def moe_route_ds(logits, bias, k: int, n_group: int, topk_group: int, method: in
   T, E = lf.shape
   if n_group > 1 and topk_group < n_group:
     g = choice.view(T, n_group, E // n_group)
-    gs = g.topk(2, -1).values.sum(-1) if method == 2 else g.max(-1).values
+    gs = g.topk(2, -1).values.sum(-1) if method == 2 and E // n_group > 1 else g.max(-1).values
     keep = torch.zeros_like(gs).scatter_(1, gs.topk(topk_group, -1).indices, 1.0)
     mask = keep[:, :, None].expand(T, n_group, E // n_group).reshape(T, E).bool()
     choice = choice.masked_fill(~mask, float("-inf"))
@@ -320,6 +320,9 @@ def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, o
   _, H, dv, d = state.shape  # stored transposed: S^T [dv, d] per head
   G = q.shape[1] // d
   rep = H // G
+  norm_ch = v.shape[1] == H * (dv - 1)  # the state's last value channel is a normaliser fed with ones; beta: input scale
+  if norm_ch:
+    dv -= 1
   for b in range(state_slots.numel()):
     t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
     if slot < 0 or t1 == t0:
@@ -329,7 +332,11 @@ def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, o
       qt = (q[t].float() * q_scale).reshape(G, d).repeat_interleave(rep, 0)
       kt = k[t].float().reshape(G, d).repeat_interleave(rep, 0)
       vt = v[t].float().reshape(H, dv)
-      if beta is not None:
+      if norm_ch:
+        vt = torch.cat([vt, torch.ones(H, 1)], 1) * beta[t].reshape(H, 1)
+        S *= decay[t].reshape(H, 1, 1)
+        S += kt[:, :, None] * vt[:, None, :]
+      elif beta is not None:
         S *= decay[t].reshape(H, 1, 1)
         u = beta[t].reshape(H, 1) * (vt - torch.einsum("hdv,hd->hv", S, kt))
         S += kt[:, :, None] * u[:, None, :]
@@ -375,6 +382,7 @@ def pool_dims(pool: int) -> int:
 def qk_norm_rope_store(P, bias, q_off, k_off, v_off, H, G, d, dv, R, pos, cos_sin, slots, eps, qk_norm, q_out, k_cache,
                        v_cache):
   T = P.shape[0]
+  Gv = v_cache.shape[1] if k_off >= 0 else G  # value heads (fewer than key heads when key heads share values)
   Pb = P.float() if bias is None else P.float() + bias.float()
   half = R // 2
 
@@ -393,7 +401,7 @@ def qk_norm_rope_store(P, bias, q_off, k_off, v_off, H, G, d, dv, R, pos, cos_si
   ok = slots >= 0
   s = slots[ok].long()
   k_cache[s // PAGE, :, s % PAGE] = prep(Pb[:, k_off:k_off + G * d].reshape(T, G, d))[ok].to(k_cache.dtype)
-  v_cache[s // PAGE, :, :, s % PAGE] = Pb[:, v_off:v_off + G * dv].reshape(T, G, dv)[ok].to(v_cache.dtype)
+  v_cache[s // PAGE, :, :, s % PAGE] = Pb[:, v_off:v_off + Gv * dv].reshape(T, Gv, dv)[ok].to(v_cache.dtype)
 
 
 def _pool_slot(blk: int, pool: int):
@@ -429,7 +437,8 @@ def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, 
     npg = -(-n // PAGE)
     pages = block_tables[b, :npg].long()
     k = k_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float()
-    v = v_cache[pages].permute(0, 3, 1, 2).reshape(npg * PAGE, G, dv)[:n].float()
+    Gv = v_cache.shape[1]  # (key heads that share a value head: G / Gv neighbours)
+    v = v_cache[pages].permute(0, 3, 1, 2).reshape(npg * PAGE, Gv, dv)[:n].float().repeat_interleave(G // Gv, 1)
     nb = n // pool if (pool and window) else 0
     if nb:
       loc = [_pool_slot(j, pool) for j in range(nb)]
@@ -505,14 +514,20 @@ def moe_weighted_sum(y, slot_of, topw, k, sh_y, P, shg_off, out, splits=1):
 
 # ------------------------------------------------------------------ sandwich blocks: latent attention, gated feed-forwards
 # Torch twins of csrc/latent.hip.
-def sandwich_add_norm(x, y, wb, wn, eps, out):
-  """x += y / rms(y) * wb in place (y None: nothing is added); with wn, out[:, :D] = x / rms(x) * wn."""
+def sandwich_add_norm(x, y, wb, wn, eps, out, bb=None, bn=None, mult=1.0):
+  """x += mult * norm(y) in place (y None: nothing is added); with wn, out[:, :D] = norm(x).  norm(v) = v / rms(v) * w,
+  or with a bias (bb / bn) the layer norm (v - mean) / sqrt(var + eps) * w + b."""
   D = x.shape[1]
+
+  def norm(v, w, b):
+    if b is None:
+      return v / torch.sqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    c = v - v.mean(-1, keepdim=True)
+    return c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float() + b.float()
   if y is not None:
-    yy = y[:, :D].float()
-    x += yy / torch.sqrt(yy.pow(2).mean(-1, keepdim=True) + eps) * wb.float()
+    x += mult * norm(y[:, :D].float(), wb, bb)
   if wn is not None:
-    out[:, :D] = (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * wn.float()).to(out.dtype)
+    out[:, :D] = norm(x, wn, bn).to(out.dtype)
 
 
 def _rope_pairs(x, cs, R, interleaved):
@@ -595,3 +610,69 @@ def glu_act(P, gate_off, up_off, Fd, clamped, limit, out):
   else:
     y = F.silu(g) * u
   out[:, :Fd] = y.to(out.dtype)
+
+
+# ------------------------------------------------------------------ layer-norm sandwich blocks: differential attention, mlstm, lightning
+# Torch twins of csrc/recurrent_gates.hip.
+def diff_attn_out(a, P, g_off, H, G, lam, post, eps, out):
+  """a [T, 2 H dv]: the two maps' attention outputs, heads ordered (kv head, map, head of the group) -> out[:, :H dv] =
+  rms_norm(a_1 - lam a_2) * post * sigmoid(P[:, g_off + head]), heads in their own order."""
+  T = a.shape[0]
+  rep = H // G
+  x = a.float().reshape(T, G, 2, rep, -1)
+  o = (x[:, :, 0] - lam * x[:, :, 1]).reshape(T, H, -1)
+  o = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps) * post
+  o = o * torch.sigmoid(P[:, g_off:g_off + H].float())[:, :, None]
+  out[:, :o.shape[1] * o.shape[2]] = o.reshape(T, -1).to(out.dtype)
+
+
+def sigmoid_gate_mul(a, P, g_off, out):
+  """out[:, :n] = a * sigmoid(P[:, g_off : +n]), n = a's row."""
+  n = a.shape[1]
+  out[:, :n] = (a.float() * torch.sigmoid(P[:, g_off:g_off + n].float())).to(out.dtype)
+
+
+def silu_cols(P, off, n, out):
+  """out [T, n] fp32 = silu(P[:, off : +n])."""
+  out.copy_(F.silu(P[:, off:off + n].float()))
+
+
+def mlstm_gates(P, i_off, f_off, gate_b, cap, mstate, state_slots, cu_q, decay, inscale, mout):
+  """Per head and token: i = cap tanh((P[i_off + h] + b_i) / cap), f = logsigmoid(cap tanh((P[f_off + h] + b_f) / cap)),
+  m_t = max(f + m_(t-1), i) from the slot's running maximum mstate [slots, H] (updated); decay = e^(f + m_(t-1) - m_t),
+  inscale = e^(i - m_t), mout = m_t, each [T, H]."""
+  H = mstate.shape[1]
+  gi = cap * torch.tanh((P[:, i_off:i_off + H].float() + gate_b[:H].float()) / cap)
+  gf = F.logsigmoid(cap * torch.tanh((P[:, f_off:f_off + H].float() + gate_b[H:].float()) / cap))
+  for b in range(state_slots.numel()):
+    t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
+    if slot < 0 or t1 == t0:
+      continue
+    m = mstate[slot].clone()
+    for t in range(t0, t1):
+      new = torch.maximum(gf[t] + m, gi[t])
+      decay[t], inscale[t], mout[t] = torch.exp(gf[t] + m - new), torch.exp(gi[t] - new), new
+      m = new
+    mstate[slot] = m
+
+
+def gated_group_norm(o, m, w, P, g_off, groups, eps, out):
+  """o [T, groups * gs] (m None) or [T, groups * (gs + 1)] with m [T, groups]: each group's last channel is then a
+  normaliser n and its values are divided by max(|n|, e^(-m)) + 1e-6 first.  out[:, :groups gs] = the values divided by
+  their group's RMS, times w [groups gs], times sigmoid(P[:, g_off : +groups gs])."""
+  T = o.shape[0]
+  x = o.float().reshape(T, groups, -1)
+  if m is not None:
+    den = torch.maximum(x[..., -1].abs(), torch.exp(-m.float())) + 1e-6
+    x = x[..., :-1] / den[..., None]
+  x = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+  n = x.shape[1] * x.shape[2]
+  out[:, :n] = (x.reshape(T, n) * w.float() * torch.sigmoid(P[:, g_off:g_off + n].float())).to(out.dtype)
+
+
+def pair_norm_mean(y1, y2, w, eps, out):
+  """out [T, D] fp32 = (y1 / rms(y1) * w[0] + y2 / rms(y2) * w[1]) / 2 (y rows may be wider than D)."""
+  D = out.shape[1]
+  a, b = y1[:, :D].float(), y2[:, :D].float()
+  out.copy_(0.5 * (a / torch.sqrt(a.pow(2).mean(-1, keepdim=True) + eps) * w[0].float() +
+                   b / torch.sqrt(b.pow(2).mean(-1, keepdim=True) + eps) * w[1].float()))
