@@ -9,6 +9,7 @@ namespace xot {
 void bind_mixers(pybind11::module& m);  // csrc/mixers.hip
 void bind_hybrid(pybind11::module& m);  // csrc/hybrid.hip
 void bind_latent(pybind11::module& m);  // csrc/latent.hip
+void bind_recurrent_gates(pybind11::module& m);  // csrc/recurrent_gates.hip
 }
 
 namespace {
@@ -1023,6 +1024,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   xot::bind_mixers(m);
   xot::bind_hybrid(m);
   xot::bind_latent(m);
+  xot::bind_recurrent_gates(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("rmsnorm_bwd", &rmsnorm_bwd, py::arg("x"), py::arg("w"), py::arg("dy"), py::arg("dx"), py::arg("dw"),
         py::arg("eps"), py::arg("res") = py::none());

@@ -56,7 +56,7 @@ template <typename AT>
 __global__ __launch_bounds__(256) void qk_norm_rope_store_k(
     const float* __restrict__ P, int ldp, const float* __restrict__ bias, int q_off, int k_off, int v_off, int H, int G,
     int d, int dv, int R, const int* __restrict__ pos, const float* __restrict__ cos_sin, const int64_t* __restrict__ slots,
-    float eps, int qk_norm, AT* __restrict__ q_out, AT* __restrict__ k_cache, AT* __restrict__ v_cache) {
+    float eps, int qk_norm, AT* __restrict__ q_out, AT* __restrict__ k_cache, AT* __restrict__ v_cache, int Gv) {
   const int t = blockIdx.x;
   const float* row = P + (int64_t)t * ldp;
   const float* cs = cos_sin + (int64_t)pos[t] * R;
@@ -100,9 +100,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_k(
     }
   }
   if (k_off >= 0 && slot >= 0) {
-    for (int e = threadIdx.x; e < G * dv; e += blockDim.x) {
+    for (int e = threadIdx.x; e < Gv * dv; e += blockDim.x) {  // (Gv value heads: G, or fewer when key heads share values)
       const int g = e / dv, i = e - g * dv;
-      const int64_t pg = (slot / PAGE_TOK) * G + g;
+      const int64_t pg = (slot / PAGE_TOK) * Gv + g;
       stf(v_cache + (pg * dv + i) * PAGE_TOK + (slot % PAGE_TOK), row[v_off + e] + (bias ? bias[v_off + e] : 0.0f));
     }
   }
@@ -153,12 +153,12 @@ __global__ void kv_pool_update_k(const AT* __restrict__ k_cache, const AT* __res
 // denominators of one); at the end the waves' (maximum, denominator, sums) are merged through LDS.
 constexpr int WATT_WAVES = 8;
 
-template <typename AT, int REP>
+template <typename AT, typename OT, int REP>
 __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
     const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache, const AT* __restrict__ kp,
     const AT* __restrict__ vp, const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int B, const float* __restrict__ sink, float scale, int window, int pool, int per,
-    AT* __restrict__ out, int ldo, int H, int G, int d, int dv) {
+    OT* __restrict__ out, int ldo, int H, int G, int d, int dv, int Gv) {
   constexpr int TILE = REP >= 8 ? 128 : 256;
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -171,6 +171,7 @@ __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
   if (ctx <= 0) return;  // padding row of a captured decode batch
   const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
   const int g = h0 / (H / G);
+  const int gv = g / (G / Gv);  // the value head of this key head (G / Gv neighbouring key heads share one)
   for (int i = threadIdx.x; i < REP * d; i += blockDim.x) qs[i] = ldf(q + ((int64_t)t * H + h0) * d + i);
   __syncthreads();
   const int* bt = block_tables + (int64_t)b * width;
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
       return k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
     });
     for (int p = a0; p < a1; p += 8) {  // 8 keys of one page per step
-      const AT* vq = v_cache + ((int64_t)bt[p / PAGE_TOK] * G + g) * dv * PAGE_TOK + (p % PAGE_TOK);
+      const AT* vq = v_cache + ((int64_t)bt[p / PAGE_TOK] * Gv + gv) * dv * PAGE_TOK + (p % PAGE_TOK);
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int i = lane + 64 * c;
@@ -745,8 +746,9 @@ void check_kv(const at::Tensor& k_cache, const at::Tensor& v_cache, at::ScalarTy
              k_cache.size(1) == G && k_cache.size(2) == PAGE_TOK && k_cache.size(3) == d,
          "k_cache must be [pages, G, 64, d] of the activations' dtype");
   MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == dt && v_cache.is_contiguous() && v_cache.dim() == 4 &&
-             v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == dv && v_cache.size(3) == PAGE_TOK,
-         "v_cache must be [pages, G, dv, 64] of the activations' dtype");
+             v_cache.size(0) == k_cache.size(0) && v_cache.size(1) >= 1 && G % v_cache.size(1) == 0 && v_cache.size(2) == dv &&
+             v_cache.size(3) == PAGE_TOK,
+         "v_cache must be [pages, Gv, dv, 64] of the activations' dtype, Gv = G or a divisor of it (key heads that share values)");
 }
 
 void qk_norm_rope_store(const at::Tensor& P, const c10::optional<at::Tensor>& bias, int64_t q_off, int64_t k_off,
@@ -755,6 +757,7 @@ void qk_norm_rope_store(const at::Tensor& P, const c10::optional<at::Tensor>& bi
                         at::Tensor& k_cache, at::Tensor& v_cache) {
   const int ldp = ld_of(P, "P");
   const int64_t T = P.size(0);
+  int64_t Gv = G;
   if (T == 0) return;
   i32c(pos, "pos");
   f32c(cos_sin, "cos_sin");
@@ -766,13 +769,14 @@ void qk_norm_rope_store(const at::Tensor& P, const c10::optional<at::Tensor>& bi
   if (k_off >= 0) {
     MCHECK(v_off >= 0, "keys without values");
     cols_ok(P, k_off, G * d, "k");
-    cols_ok(P, v_off, G * dv, "v");
     check_kv(k_cache, v_cache, q_out.scalar_type(), G, d, dv);
+    Gv = v_cache.size(1);
+    cols_ok(P, v_off, Gv * dv, "v");
   }
   const float* bp = nullptr;
   if (bias.has_value()) {
     f32c(*bias, "bias");
-    MCHECK(bias->numel() >= std::max(q_off + H * d, std::max(k_off + G * d, v_off + G * dv)), "bias must cover the q / k / v columns");
+    MCHECK(bias->numel() >= std::max(q_off + H * d, std::max(k_off + G * d, v_off + Gv * dv)), "bias must cover the q / k / v columns");
     bp = bias->data_ptr<float>();
   }
   MCHECK(q_out.is_cuda() && is_act(q_out) && q_out.is_contiguous() && q_out.numel() == T * H * d, "q_out must be [T, H, d]");
@@ -782,12 +786,12 @@ void qk_norm_rope_store(const at::Tensor& P, const c10::optional<at::Tensor>& bi
     qk_norm_rope_store_k<uint16_t><<<T, 256, 0, stream()>>>(
         P.data_ptr<float>(), ldp, bp, (int)q_off, (int)k_off, (int)v_off, (int)H, (int)G, (int)d, (int)dv, (int)R,
         pos.data_ptr<int>(), cos_sin.data_ptr<float>(), slots.data_ptr<int64_t>(), (float)eps, (int)qk_norm,
-        (uint16_t*)q_out.data_ptr(), (uint16_t*)k_cache.data_ptr(), (uint16_t*)v_cache.data_ptr());
+        (uint16_t*)q_out.data_ptr(), (uint16_t*)k_cache.data_ptr(), (uint16_t*)v_cache.data_ptr(), (int)Gv);
   else
     qk_norm_rope_store_k<float><<<T, 256, 0, stream()>>>(
         P.data_ptr<float>(), ldp, bp, (int)q_off, (int)k_off, (int)v_off, (int)H, (int)G, (int)d, (int)dv, (int)R,
         pos.data_ptr<int>(), cos_sin.data_ptr<float>(), slots.data_ptr<int64_t>(), (float)eps, (int)qk_norm,
-        q_out.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>());
+        q_out.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(), (int)Gv);
 }
 
 void check_pools(const at::Tensor& k_cache, const at::Tensor& kp, const at::Tensor& vp, int64_t pool, int64_t G, int64_t d,
@@ -808,6 +812,7 @@ void kv_pool_update(const at::Tensor& k_cache, const at::Tensor& v_cache, at::Te
   MCHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && is_act(k_cache), "caches must be 4-D bf16 / fp32");
   const int64_t G = k_cache.size(1), d = k_cache.size(3), dv = v_cache.size(2), B = ctx_lens.numel();
   check_kv(k_cache, v_cache, k_cache.scalar_type(), G, d, dv);
+  MCHECK(v_cache.size(1) == G, "pooled blocks need a value head per key head");
   int per;
   check_pools(k_cache, kp, vp, pool, G, d, dv, &per);
   i32c(block_tables, "block_tables");
@@ -869,9 +874,12 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
     MCHECK(sink->numel() == H, "sink must hold one logit per head");
     sp = sink->data_ptr<float>();
   }
-  MCHECK(out.scalar_type() == q.scalar_type(), "out must have q's dtype");
+  const int64_t Gv = v_cache.size(1);
+  MCHECK(out.scalar_type() == q.scalar_type() || out.scalar_type() == at::kFloat, "out must have q's dtype or be fp32");
+  MCHECK(!pooled || Gv == G, "pooled blocks need a value head per key head");
   const int ldo = act_ld(out, T, H * dv, "out");
-  if (q.scalar_type() == at::kBFloat16 && max_qlen >= 16 && d == dv && (d == 32 || d == 64 || d == 128) && ldo % 4 == 0 &&
+  const bool o32 = out.scalar_type() == at::kFloat;
+  if (q.scalar_type() == at::kBFloat16 && !o32 && Gv == G && max_qlen >= 16 && d == dv && (d == 32 || d == 64 || d == 128) && ldo % 4 == 0 &&
       WATT_MFMA) {
     const dim3 grid((unsigned)B, (unsigned)((max_qlen + 127) / 128), (unsigned)H);
     const uint16_t* kpp = pooled ? (const uint16_t*)kp->data_ptr() : nullptr;
@@ -898,23 +906,26 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
   while (rep > 1 && (lds_of(rep) > 60 * 1024 || T * (H / rep) < 256)) rep /= 2;
   const dim3 grid((unsigned)T, (unsigned)(H / rep));
   const size_t lds = lds_of(rep);
-#define WATT_GO(AT, R)                                                                                                     \
-  attn_window_pool_k<AT, R><<<grid, 64 * WATT_WAVES, lds, stream()>>>(                                                     \
+#define WATT_GO(AT, OT, R)                                                                                                 \
+  attn_window_pool_k<AT, OT, R><<<grid, 64 * WATT_WAVES, lds, stream()>>>(                                                 \
       (const AT*)q.data_ptr(), (const AT*)k_cache.data_ptr(), (const AT*)v_cache.data_ptr(),                               \
       pooled ? (const AT*)kp->data_ptr() : nullptr, pooled ? (const AT*)vp->data_ptr() : nullptr,                          \
       block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp, \
-      (float)scale, (int)window, pooled ? (int)pool : 0, per, (AT*)out.data_ptr(), ldo, (int)H, (int)G, (int)d, (int)dv)
-#define WATT_REP(AT)                   \
-  switch (rep) {                       \
-    case 8: WATT_GO(AT, 8); break;     \
-    case 4: WATT_GO(AT, 4); break;     \
-    case 2: WATT_GO(AT, 2); break;     \
-    default: WATT_GO(AT, 1); break;    \
+      (float)scale, (int)window, pooled ? (int)pool : 0, per, (OT*)out.data_ptr(), ldo, (int)H, (int)G, (int)d, (int)dv,  \
+      (int)Gv)
+#define WATT_REP(AT, OT)                   \
+  switch (rep) {                           \
+    case 8: WATT_GO(AT, OT, 8); break;     \
+    case 4: WATT_GO(AT, OT, 4); break;     \
+    case 2: WATT_GO(AT, OT, 2); break;     \
+    default: WATT_GO(AT, OT, 1); break;    \
   }
-  if (q.scalar_type() == at::kBFloat16) {
-    WATT_REP(uint16_t)
+  if (q.scalar_type() == at::kBFloat16 && o32) {
+    WATT_REP(uint16_t, float)
+  } else if (q.scalar_type() == at::kBFloat16) {
+    WATT_REP(uint16_t, uint16_t)
   } else {
-    WATT_REP(float)
+    WATT_REP(float, float)
   }
 #undef WATT_REP
 #undef WATT_GO

@@ -1,6 +1,7 @@
 // Kernels of sandwich-block models with latent attention (fp32 residual stream; activations AT = bf16 or fp32).
 //
-//   sandwich_add_norm   x += rms_norm(y) * wb, and the next sublayer's input rms_norm(x) * wn in the GEMM operand dtype
+//   sandwich_add_norm   x += mult * norm(y), and the next sublayer's input norm(x) in the GEMM operand dtype (RMS norms with
+//                       a weight, or layer norms with weight and bias)
 //   latent_kv_store     kv latent RMS norm + RoPE of the shared rotated key part -> one cache row per token; the query
 //                       latent's RMS norm
 //   latent_q_rope       queries: unrotated parts per head [H, T, dn] (operand of q . W_uk), rotated parts after RoPE
@@ -27,27 +28,44 @@ __device__ __forceinline__ s16x4 tr_read(const uint16_t* p) {
 constexpr float LOG2E_F = 1.4426950408889634f;
 
 // ------------------------------------------------------------------ residual add of a normed sublayer result + next norm
+// norm of one row held in global memory: v / rms(v) * w, or with a bias the layer norm (v - mean) / sqrt(var + eps) * w + b
+// (the variance as the mean of the squared deviations, in a pass of its own).  Returns (shift, scale).
+__device__ __forceinline__ void row_norm_stats(const float* v, int D, bool center, float eps, float* red, float* shift,
+                                               float* scale) {
+  float mean = 0.0f;
+  if (center) {
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) s += v[i];
+    mean = block_sum(s, red) / D;
+  }
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float c = v[i] - mean;
+    ss += c * c;
+  }
+  ss = block_sum(ss, red);
+  *shift = mean;
+  *scale = 1.0f / sqrtf(ss / D + eps);
+}
+
 template <typename AT>
 __global__ __launch_bounds__(256) void sandwich_add_norm_k(float* __restrict__ x, const float* __restrict__ y, int ldy,
-                                                           const float* __restrict__ wb, const float* __restrict__ wn,
-                                                           float eps, AT* __restrict__ out, int ldo, int D) {
+                                                           const float* __restrict__ wb, const float* __restrict__ bb,
+                                                           const float* __restrict__ wn, const float* __restrict__ bn,
+                                                           float mult, float eps, AT* __restrict__ out, int ldo, int D) {
   __shared__ float red[8];
   const int64_t t = blockIdx.x;
   float* xr = x + t * D;
   if (y) {
     const float* yr = y + t * ldy;
-    float ss = 0.0f;
-    for (int i = threadIdx.x; i < D; i += blockDim.x) ss += yr[i] * yr[i];
-    ss = block_sum(ss, red);
-    const float r = 1.0f / sqrtf(ss / D + eps);
-    for (int i = threadIdx.x; i < D; i += blockDim.x) xr[i] += yr[i] * r * wb[i];
+    float mu, r;
+    row_norm_stats(yr, D, bb != nullptr, eps, red, &mu, &r);
+    for (int i = threadIdx.x; i < D; i += blockDim.x) xr[i] += mult * ((yr[i] - mu) * r * wb[i] + (bb ? bb[i] : 0.0f));
   }
   if (wn) {  // (a thread re-reads the elements it wrote itself)
-    float ss = 0.0f;
-    for (int i = threadIdx.x; i < D; i += blockDim.x) ss += xr[i] * xr[i];
-    ss = block_sum(ss, red);
-    const float r = 1.0f / sqrtf(ss / D + eps);
-    for (int i = threadIdx.x; i < D; i += blockDim.x) stf(out + t * ldo + i, xr[i] * r * wn[i]);
+    float mu, r;
+    row_norm_stats(xr, D, bn != nullptr, eps, red, &mu, &r);
+    for (int i = threadIdx.x; i < D; i += blockDim.x) stf(out + t * ldo + i, (xr[i] - mu) * r * wn[i] + (bn ? bn[i] : 0.0f));
   }
 }
 
@@ -547,13 +565,24 @@ __global__ __launch_bounds__(256) void latent_attn_merge_k(const float* __restri
 const bool LATT_MFMA = []() { const char* e = getenv("XOT_LATT_MFMA"); return !(e && e[0] == '0'); }();
 
 void sandwich_add_norm(at::Tensor& x, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& wb,
-                       const c10::optional<at::Tensor>& wn, double eps, const c10::optional<at::Tensor>& out) {
+                       const c10::optional<at::Tensor>& wn, double eps, const c10::optional<at::Tensor>& out,
+                       const c10::optional<at::Tensor>& bb, const c10::optional<at::Tensor>& bn, double mult) {
   f32c(x, "x");
   MCHECK(x.dim() == 2, "x must be [T, D]");
   const int64_t T = x.size(0), D = x.size(1);
   if (T == 0) return;
-  const float *yp = nullptr, *bp = nullptr, *np = nullptr;
+  const float *yp = nullptr, *bp = nullptr, *np = nullptr, *bbp = nullptr, *bnp = nullptr;
   int ldy = 0, ldo = 0;
+  if (bb.has_value()) {
+    f32c(*bb, "bb");
+    MCHECK(bb->numel() == D && y.has_value(), "the result norm's bias must hold D numbers");
+    bbp = bb->data_ptr<float>();
+  }
+  if (bn.has_value()) {
+    f32c(*bn, "bn");
+    MCHECK(bn->numel() == D && wn.has_value(), "the next norm's bias must hold D numbers");
+    bnp = bn->data_ptr<float>();
+  }
   if (y.has_value()) {
     ldy = ld_of(*y, "y");
     MCHECK(y->size(0) == T && y->size(1) >= D && wb.has_value(), "the sublayer's result must be fp32 [T, >= D] rows with a norm weight");
@@ -574,9 +603,11 @@ void sandwich_add_norm(at::Tensor& x, const c10::optional<at::Tensor>& y, const 
   }
   if (!yp && !np) return;
   if (bf)
-    sandwich_add_norm_k<uint16_t><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, np, (float)eps, (uint16_t*)op, ldo, (int)D);
+    sandwich_add_norm_k<uint16_t><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, bbp, np, bnp, (float)mult, (float)eps,
+                                                           (uint16_t*)op, ldo, (int)D);
   else
-    sandwich_add_norm_k<float><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, np, (float)eps, (float*)op, ldo, (int)D);
+    sandwich_add_norm_k<float><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, bbp, np, bnp, (float)mult, (float)eps,
+                                                        (float*)op, ldo, (int)D);
 }
 
 void check_rope(const at::Tensor& pos, const at::Tensor& cos_sin, int64_t T, int64_t rot, int64_t dr) {

@@ -556,7 +556,9 @@ __global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int
 // while the current one is consumed.
 // MODE 1 (delta rule): S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   MODE 0: S = diag(a) S + k v^T; o = S^T q
 // (a decay per key channel).   MODE 2: S = g S + k v^T; o = S^T q (one decay per head: the state-space-duality form
-// with k = B, q = C, v = dt x).
+// with k = B, q = C, v = dt x).   MODE 3: MODE 2 with an input scale b per head and token and a normaliser: the state has
+// one value channel more than v (dvin + 1), fed with ones, S = g S + k (b [v | 1])^T, so the last channel is n = g n + b k
+// and the last output n . q (the stabilised matrix memory of xLSTM, g and b computed by its gate kernel).
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
   const int m = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
@@ -577,10 +579,10 @@ template <int KR, int RS, int MODE>
 __global__ __launch_bounds__(256) void linear_recurrence_k(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
-    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv, int dvin,
     float* __restrict__ out) {
   constexpr int DP = KR * RS;  // padded key dim
-  constexpr bool DELTA = MODE == 1, SCALAR = MODE != 0;
+  constexpr bool DELTA = MODE == 1, SCALAR = MODE != 0, NORMCH = MODE == 3;
   constexpr int COLS = 256 / RS;
   constexpr int TB = DP >= 256 ? 8 : 16;
   constexpr int NQ = TB * DP / 256, NV = (TB * COLS + 255) / 256;
@@ -626,11 +628,12 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int e = tid + 256 * j, tt = e / COLS, c = cb * COLS + e % COLS;
-      pv[j] = (e < TB * COLS && c < dv && tb + tt < n) ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
+      pv[j] = (e < TB * COLS && c < dvin && tb + tt < n) ? v[(int64_t)(t0 + tb + tt) * ldv + h * dvin + c] : 0.0f;
+      if (NORMCH && e < TB * COLS && c == dvin && tb + tt < n) pv[j] = 1.0f;
     }
     if (SCALAR && tid < TB && tb + tid < n) {
       pg0 = decay[(int64_t)(t0 + tb + tid) * H + h];
-      if (DELTA) pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
+      if (DELTA || NORMCH) pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
     }
   };
   auto stage = [&](int buf) {  // registers -> LDS
@@ -661,7 +664,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
     if (more) fetch(tb + TB);
 #pragma unroll 2
     for (int tt = 0; tt < nt; ++tt) {
-      const float vc = sv[buf][tt][cl];
+      const float vc = NORMCH ? sv[buf][tt][cl] * sg[buf][tt][1] : sv[buf][tt][cl];
       float kk[KR], qq[KR];
 #pragma unroll
       for (int m = 0; m < KR; ++m) {
@@ -989,11 +992,11 @@ void gla_prep(const at::Tensor& P, int64_t a1_off, const at::Tensor& a2, const a
 template <int RS, int MODE>
 void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay,
                 const float* beta, float q_scale, float* state, const int* slots, const int* cu, int H, int G, int d, int dv,
-                float* out) {
+                int dvin, float* out) {
 #define REC_CASE(DPAD)                                                                                                 \
   case DPAD:                                                                                                           \
     linear_recurrence_k<DPAD / RS, RS, MODE><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, \
-                                                                          state, slots, cu, H, G, d, dv, out);         \
+                                                                          state, slots, cu, H, G, d, dv, dvin, out);   \
     break;
   switch (KR * RS) {  // padded key dim
     REC_CASE(16)
@@ -1009,7 +1012,8 @@ void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int 
 
 // q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta rule, or
 // without beta: one decay per head and a plain outer-product write) or [T, H d] (per key channel); beta [T, H] (delta
-// only).  state [slots, H, dv, d] (S^T: key rows contiguous).
+// only; an input scale for a state with a normaliser channel: then v is [T, H (dv - 1)]).  state [slots, H, dv, d] (S^T: key
+// rows contiguous).
 void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& decay,
                        const c10::optional<at::Tensor>& beta, double q_scale, at::Tensor& state, const at::Tensor& state_slots,
                        const at::Tensor& cu_q, at::Tensor& out) {
@@ -1024,17 +1028,20 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   if (T == 0 || B == 0) return;
   MCHECK(q.size(1) % d == 0 && q.size(1) == k.size(1), "q / k must be [T, G d]");
   const int64_t G = q.size(1) / d;
-  MCHECK(G > 0 && H % G == 0 && k.size(0) == T && v.size(0) == T && v.size(1) == H * dv && out.numel() == T * H * dv,
+  const bool normch = v.size(1) == H * (dv - 1);  // the state's last value channel is a normaliser, beta an input scale
+  const int64_t dvin = normch ? dv - 1 : dv;
+  MCHECK(G > 0 && H % G == 0 && k.size(0) == T && v.size(0) == T && v.size(1) == H * dvin && out.numel() == T * H * dv,
          "linear_recurrence: shape mismatch");
   MCHECK(cu_q.numel() == B + 1, "cu_q must hold B + 1 offsets");
-  const bool delta = beta.has_value();
-  if (delta) {
+  MCHECK(!normch || beta.has_value(), "a state with a normaliser channel needs the input scales");
+  const bool delta = beta.has_value() && !normch;
+  if (beta.has_value()) {
     f32c(*beta, "beta");
     MCHECK(beta->numel() == T * H && decay.numel() == T * H, "delta rule: beta / decay must be [T, H]");
   } else if (decay.numel() != T * H) {
     MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
   }
-  const bool scalar = !delta && decay.numel() == T * H;  // one decay per head, q / k shared by H / G heads
+  const bool scalar = !delta && !normch && decay.numel() == T * H;  // one decay per head, q / k shared by H / G heads
   int DP = 16;
   while (DP < d) DP *= 2;
   MCHECK(DP <= 256, "linear_recurrence: key dim above 256");
@@ -1043,12 +1050,12 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   const int RS = 16;
   const int cols = 256 / RS;
   const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + cols - 1) / cols));
-  const float* bp = delta ? beta->data_ptr<float>() : nullptr;
+  const float* bp = beta.has_value() ? beta->data_ptr<float>() : nullptr;
 #define REC_GO(R, D)                                                                                                          \
   launch_rec<R, D>(DP / R, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,              \
                    decay.data_ptr<float>(), bp, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),        \
-                   cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>())
-  if (delta) REC_GO(16, 1); else if (scalar) REC_GO(16, 2); else REC_GO(16, 0);
+                   cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, (int)dvin, out.data_ptr<float>())
+  if (delta) REC_GO(16, 1); else if (normch) REC_GO(16, 3); else if (scalar) REC_GO(16, 2); else REC_GO(16, 0);
 #undef REC_GO
 }
 

@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void moe_topk_ds_kernel(const float* __restric
     for (int i = 0; i < MOE_DS_EPL; ++i) sc[i] /= den;
   } else {
 #pragma unroll
-    for (int i = 0; i < MOE_DS_EPL; ++i) sc[i] = lane + 64 * i < E ? 1.f / (1.f + __expf(-sc[i])) : 0.f;
+    for (int i = 0; i < MOE_DS_EPL; ++i) sc[i] = lane + 64 * i < E ? 1.f / (1.f + expf(-sc[i])) : 0.f;
   }
 #pragma unroll
   for (int i = 0; i < MOE_DS_EPL; ++i) {
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void moe_topk_ds_kernel(const float* __restric
           b2 = v;
         }
       }
-      gsc = method == 2 ? a + b2 : a;
+      gsc = (method == 2 && per > 1) ? a + b2 : a;  // (a group of one expert has no second best)
     }
     keep = 0;
     for (int j = 0; j < topk_group; ++j) {  // wave argmax over the groups (ties: lower group id)

@@ -121,8 +121,10 @@ class KVCache:
         src = i if a.kv_from < 0 else a.kv_from
         if src not in ids:
           raise ValueError(f"layer {i} reads the keys and values of layer {src}, which is not on this shard")
-        js = ids.index(src)
+        # (the source's run that this run follows: a looped layer has a cache of its own in every pass)
+        js = j if src == i else max([jj for jj in range(j) if ids[jj] == src], default=ids.index(src))
         self.k[j], self.v[j] = self.k[js], self.v[js]
+        src = js  # pooled caches belong to the run, too
         if a.pool > 0 and a.window > 0:
           if (src, a.pool) not in made:
             per = K.pool_dims(a.pool)
@@ -143,13 +145,16 @@ class KVCache:
     if c.is_mixed:
       ids = [i for i, _ in c.layer_runs(layer_ids if layer_ids is not None else range(n_layers))]
       n, seen = 0, set()
-      for i in ids:
+      for j, i in enumerate(ids):
         a, w = c.layer_specs[i].kv_dims, c.layer_specs[i].wattn
         if a is not None:
           n += PAGE * (a[0] * a[1] + (a[3] if len(a) > 3 else a[0]) * a[2]) * itemsize
-        if w is not None and w.pool > 0 and w.window > 0 and (w.kv_from if w.kv_from >= 0 else i, w.pool) not in seen:
-          seen.add((w.kv_from if w.kv_from >= 0 else i, w.pool))
-          n += w.kv_heads * K.pool_dims(w.pool) * (w.dim + w.vdim) * itemsize
+        if w is not None and w.pool > 0 and w.window > 0:
+          # (pooled caches: one per run of the source layer and block size)
+          js = j if w.kv_from < 0 else max([jj for jj in range(j) if ids[jj] == w.kv_from], default=-1)
+          if (js, w.pool) not in seen:
+            seen.add((js, w.pool))
+            n += w.kv_heads * K.pool_dims(w.pool) * (w.dim + w.vdim) * itemsize
       return max(1, n)
     if c.is_mla:
       return n_layers * PAGE * c.mla_dim * 2
