@@ -185,6 +185,34 @@ def latent_configs(name: str):
   return latent, ds
 
 
+def memory_configs(name: str):
+  """(Kopalorn-design config, the closest existing model: the Mogelix-design stack of equal width and depth, whose window
+  attention, linear recurrence and relu^2 experts run on the same kernels).  Kopalorn layers in turn: differential
+  attention (two maps of half the head size over values of the full head size, the size's chunk as sliding window);
+  mlstm (one head per attention head, key and value size of the head); causal gated attention beside lightning
+  attention of half as many heads.  Every layer sits under 8 relu^2 experts of half the dense ff in 4 groups (2 kept, 2
+  chosen) plus a shared expert of 1024.  No loop (equal depth on both sides)."""
+  from xotorch_support_jetson_amd.models.config import from_hf_config
+  z = MIXER_SIZES[name]
+  H, G, d, chunk, rot = z["attn"]
+  W = z["width"]
+  moe = {"kind": "moe", "expert": {"ff": (z["ff"] // 2 + 127) // 128 * 128}, "shared": {"ff": 1024},
+         "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+  hr = max(H // 2, 1)
+  kinds = [
+    {"type": "attention", "mlp": moe,
+     "mixer": {"heads": H, "kv_heads": G, "dim": d // 2, "vdim": d, "diff": 0.8, "scale": (d // 2) ** -0.5, "mask": {"size": chunk},
+               "rot": {"base": 1e6, "dims": min(rot, d // 2)}}},
+    {"type": "mlstm", "mlp": moe, "mixer": {"heads": H, "dim": d, "vdim": d, "gate_cap": 15.0}},
+    {"type": "parallel", "mlp": moe,
+     "mixer": {"left": {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "scale": d ** -0.5},
+               "right": {"heads": hr, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** -(5 + 4 * i / max(hr - 1, 1)) for i in range(hr)]}}},
+  ]
+  memory = from_hf_config({"architecture": "Kopalorn", "vocab": 32000, "width": W, "norm": {"eps": 1e-5}, "residual_mult": 0.5,
+                           "layers": [kinds[i % 3] for i in range(z["layers"])]})
+  return memory, hybrid_configs(name)[0]
+
+
 def bench_mixers(args, sizes=None, kinds=("tarepel", "llama"), configs=mixer_configs,
                  what="Tarepel-design layers beside a Llama-style stack of equal size"):
   """Prefill and decode throughput of mixed-layer designs at sizes like a real model's (random weights), beside
@@ -266,7 +294,11 @@ def main():
                   help="instead of the headline: Nenizen-design layers (latent attention with window / sink / output "
                        "gates, clamped gated feed-forward, SiLU experts) beside a DeepSeek-V2-style stack of the same "
                        "latent sizes at the named sizes; one GPU")
-  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers / --hybrid / --latent: sequences per step")
+  ap.add_argument("--memory", default=None, metavar="SIZES",
+                  help="instead of the headline: Kopalorn-design layers (differential window attention, mlstm, gated "
+                       "attention beside lightning attention, relu^2 experts with grouped sigmoid routing) beside the "
+                       "Mogelix-design stack at the named sizes; one GPU")
+  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers / --hybrid / --latent / --memory: sequences per step")
   args = ap.parse_args()
   os.environ["XOT_WEIGHT_DTYPE"] = args.weight_dtype
   if args.mixers:
@@ -278,6 +310,10 @@ def main():
   if args.latent:
     return bench_mixers(args, args.latent, ("nenizen", "deepseek"), latent_configs,
                         "Nenizen-design layers beside a DeepSeek-V2-style stack of equal size")
+
+  if args.memory:
+    return bench_mixers(args, args.memory, ("kopalorn", "mogelix"), memory_configs,
+                        "Kopalorn-design layers beside a Mogelix-design stack of equal size")
 
   from xotorch_support_jetson_amd.models.config import preset
   from xotorch_support_jetson_amd.parallel.comm import P2PTransport, init_distributed

@@ -333,7 +333,7 @@ __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
   }
 }
 
-// MFMA kernel (bf16, d = dv = 32 NK): a workgroup owns 128 consecutive queries of one (sequence, head), 32 per wave, and
+// MFMA kernel (bf16 caches; key size 32 NK, value size 32 NV; output bf16 or fp32): a workgroup owns 128 consecutive queries of one (sequence, head), 32 per wave, and
 // walks first the pooled blocks that its last query sees, then the tokens from its first query's window on, a tile of
 // KT keys at a time: the K rows and V^T runs of the tile are staged in LDS and shared by the four waves (pooled
 // entries are gathered row by row and their values transposed on the way in).  Scores are computed transposed,
@@ -342,17 +342,18 @@ __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
 // denominators), and the exponentials, rounded to bf16, are as they lie the B operand of O^T += V^T P^T, whose k slots
 // (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.  Scores, maxima and sums are fp32 (base-2
 // exponentials of scores scaled by log2 e); the sink's logit starts the running maximum with a denominator of one.
-template <int NK>
+template <int NK, int NV, typename OT>
 __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const uint16_t* __restrict__ kp, const uint16_t* __restrict__ vp, const int* __restrict__ block_tables, int width,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, const float* __restrict__ sink, float scale, int window,
-    int pool, int per, uint16_t* __restrict__ out, int ldo, int H, int G) {
-  constexpr int D = NK * 32, ND = NK * 2, QT = 2;
-  constexpr int KT = D > 192 ? 32 : 64;  // keys per tile (a page holds a whole number of tiles)
+    int pool, int per, OT* __restrict__ out, int ldo, int H, int G, int Gv) {
+  // key size D = 32 NK, value size DV = 32 NV (pooled blocks: NK == NV); G / Gv neighbouring key heads share a value head
+  constexpr int D = NK * 32, DV = NV * 32, ND = NV * 2, QT = 2;
+  constexpr int KT = (D > 192 || DV > 192) ? 32 : 64;  // keys per tile (a page holds a whole number of tiles)
   constexpr int KP = D + 8, VP = KT + 8;
   constexpr float L2E = 1.4426950408889634f;
-  __shared__ __attribute__((aligned(16))) uint16_t sK[KT][KP], sV[D][VP];
+  __shared__ __attribute__((aligned(16))) uint16_t sK[KT][KP], sV[DV][VP];
   const int b = blockIdx.x, h = blockIdx.z;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, c = l & 15, g4 = l >> 4;
   const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0, ctx = ctx_lens[b];
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
   const bool active = q0 < qlen;
   const int nq = active ? min(32, qlen - q0) : 0;
   const int pos0 = ctx - qlen + q0;  // position of the wave's first query
-  const int gk = h / (H / G);
+  const int gk = h / (H / G), gv = gk / (G / Gv);
   // pooled blocks a query at position p sees: those that end at or before p - window
   auto blocks_seen = [&](int p) { return (pool > 0 && p - window + 1 >= pool) ? (p - window + 1) / pool : 0; };
   s16x8 qf[QT][NK];
@@ -391,7 +392,8 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
   const int wpos0 = ctx - qlen + wq0;
   const int last = active ? pos0 + nq - 1 : -1;                  // the wave's last query
   constexpr int NCHUNK = KT * (D / 8), NCH = (NCHUNK + 255) / 256;
-  s16x8 rk[NCH], rv[NCH];
+  constexpr int NCHUNKV = KT * (DV / 8), NCHV = (NCHUNKV + 255) / 256;
+  s16x8 rk[NCH], rv[NCHV];
 
   // one staged tile: scores, mask, running softmax, O^T += V^T P^T.  pooled: key index = block index.
   auto consume = [&](int tb, bool pooled) {
@@ -472,7 +474,7 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
   };
 
   // ---- pooled blocks [0, nbw): rows gathered from the pages that hold them, values transposed into sV
-  const int nbw = blocks_seen(wlast);
+  const int nbw = NK == NV ? blocks_seen(wlast) : 0;
   for (int tb = 0; tb < nbw; tb += KT) {
     __syncthreads();  // the previous tile has been consumed
 #pragma unroll
@@ -495,7 +497,7 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
   // ---- tokens from the first query's window on
   const int t_lo = (window > 0 ? max(0, wpos0 - window + 1) : 0) & ~(KT - 1);
   auto fetch = [&](int tb) {
-    const int64_t pg = (int64_t)bt[tb >> 6] * G + gk;
+    const int64_t pg = (int64_t)bt[tb >> 6] * G + gk, pgv = (int64_t)bt[tb >> 6] * Gv + gv;
     const int koff = tb & 63;
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
@@ -503,8 +505,13 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
       if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
       const int row = ch / (D / 8), cc = ch - row * (D / 8);
       rk[j] = ld16(k_cache + ((pg * PAGE_TOK) + koff + row) * D + cc * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < NCHV; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNKV % 256 != 0 && ch >= NCHUNKV) break;
       const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
-      rv[j] = ld16(v_cache + (pg * D + vrow) * PAGE_TOK + koff + vc * 8);
+      rv[j] = ld16(v_cache + (pgv * DV + vrow) * PAGE_TOK + koff + vc * 8);
     }
   };
   fetch(t_lo);
@@ -516,6 +523,11 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
       if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
       const int row = ch / (D / 8), cc = ch - row * (D / 8);
       st16(&sK[row][cc * 8], rk[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < NCHV; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNKV % 256 != 0 && ch >= NCHUNKV) break;
       const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
       st16(&sV[vrow][vc * 8], rv[j]);
     }
@@ -530,13 +542,17 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
     ls += __shfl_xor(ls, 32, 64);
     if (qt * 16 + c >= nq) continue;
     const float inv = ls > 0.0f ? 1.0f / ls : 0.0f;
-    uint16_t* op = out + (int64_t)(t0 + q0 + qt * 16 + c) * ldo + h * D + 4 * g4;
+    OT* op = out + (int64_t)(t0 + q0 + qt * 16 + c) * ldo + h * DV + 4 * g4;
 #pragma unroll
     for (int db = 0; db < ND; ++db) {
-      s16x4 w;
+      if constexpr (sizeof(OT) == 4) {
+        *reinterpret_cast<f32x4*>(op + db * 16) = f32x4{o[qt][db][0] * inv, o[qt][db][1] * inv, o[qt][db][2] * inv, o[qt][db][3] * inv};
+      } else {
+        s16x4 w;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) w[r] = (short)f2bf(o[qt][db][r] * inv);
-      *reinterpret_cast<s16x4*>(op + db * 16) = w;
+        for (int r = 0; r < 4; ++r) w[r] = (short)f2bf(o[qt][db][r] * inv);
+        *reinterpret_cast<s16x4*>(op + db * 16) = w;
+      }
     }
   }
 }
@@ -834,14 +850,14 @@ void kv_pool_update(const at::Tensor& k_cache, const at::Tensor& v_cache, at::Te
         per, (int)G, (int)d, (int)dv);
 }
 
-template <int NK>
+template <int NK, int NV, typename OT>
 void launch_wattn_mfma(dim3 grid, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache, const uint16_t* kp,
                        const uint16_t* vp, const at::Tensor& block_tables, const at::Tensor& cu_q, const at::Tensor& ctx_lens,
                        const float* sink, float scale, int window, int pool, int per, at::Tensor& out, int ldo, int H, int G) {
-  attn_window_pool_mfma_k<NK><<<grid, 256, 0, stream()>>>(
+  attn_window_pool_mfma_k<NK, NV, OT><<<grid, 256, 0, stream()>>>(
       (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(), kp, vp,
       block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), sink, scale,
-      window, pool, per, (uint16_t*)out.data_ptr(), ldo, H, G);
+      window, pool, per, (OT*)out.data_ptr(), ldo, H, G, (int)v_cache.size(1));
 }
 
 // max_qlen: the longest run of new tokens of one sequence in this step (below 16: single decoded tokens and short
@@ -879,21 +895,26 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
   MCHECK(!pooled || Gv == G, "pooled blocks need a value head per key head");
   const int ldo = act_ld(out, T, H * dv, "out");
   const bool o32 = out.scalar_type() == at::kFloat;
-  if (q.scalar_type() == at::kBFloat16 && !o32 && Gv == G && max_qlen >= 16 && d == dv && (d == 32 || d == 64 || d == 128) && ldo % 4 == 0 &&
-      WATT_MFMA) {
+  // the MFMA kernel: bf16 caches, runs of 16 tokens or more, value size = key size in {32, 64, 128} (bf16 or fp32 output)
+  // or twice the key size in {32, 64} with fp32 output (differential attention's maps); pooled blocks need equal sizes
+  const bool same = d == dv && (d == 32 || d == 64 || d == 128), twice = dv == 2 * d && (d == 32 || d == 64) && o32 && !pooled;
+  if (q.scalar_type() == at::kBFloat16 && max_qlen >= 16 && (same || twice) && ldo % 4 == 0 && WATT_MFMA) {
     const dim3 grid((unsigned)B, (unsigned)((max_qlen + 127) / 128), (unsigned)H);
     const uint16_t* kpp = pooled ? (const uint16_t*)kp->data_ptr() : nullptr;
     const uint16_t* vpp = pooled ? (const uint16_t*)vp->data_ptr() : nullptr;
     const int pl = pooled ? (int)pool : 0;
-    if (d == 32)
-      launch_wattn_mfma<1>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
-                           per, out, ldo, (int)H, (int)G);
-    else if (d == 64)
-      launch_wattn_mfma<2>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
-                           per, out, ldo, (int)H, (int)G);
-    else
-      launch_wattn_mfma<4>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
-                           per, out, ldo, (int)H, (int)G);
+#define WATT_MFMA_GO(NK, NV, OT)                                                                                            \
+  launch_wattn_mfma<NK, NV, OT>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale,       \
+                                (int)window, pl, per, out, ldo, (int)H, (int)G)
+    if (twice && d == 32) WATT_MFMA_GO(1, 2, float);
+    else if (twice) WATT_MFMA_GO(2, 4, float);
+    else if (d == 32 && o32) WATT_MFMA_GO(1, 1, float);
+    else if (d == 32) WATT_MFMA_GO(1, 1, uint16_t);
+    else if (d == 64 && o32) WATT_MFMA_GO(2, 2, float);
+    else if (d == 64) WATT_MFMA_GO(2, 2, uint16_t);
+    else if (o32) WATT_MFMA_GO(4, 4, float);
+    else WATT_MFMA_GO(4, 4, uint16_t);
+#undef WATT_MFMA_GO
     return;
   }
   // query heads of one kv head share a workgroup (each key row and value run is loaded once for all of them)

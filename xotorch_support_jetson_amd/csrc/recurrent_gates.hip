@@ -34,13 +34,14 @@ __global__ void diff_attn_out_k(const float* __restrict__ a, const float* __rest
   for (int i = lane; i < dv; i += 64) stf(out + (int64_t)t * ldo + h * dv + i, (a1[i] - lam * a2[i]) * k);
 }
 
-template <typename AT>
-__global__ void sigmoid_gate_mul_k(const float* __restrict__ a, const float* __restrict__ P, int ldp, int g_off, int n,
-                                   AT* __restrict__ out, int ldo, int64_t total) {
+// (a and out may be the same rows: every element is read and written by one thread)
+template <typename IT, typename AT>
+__global__ void sigmoid_gate_mul_k(const IT* a, int lda, const float* __restrict__ P, int ldp, int g_off, int n, AT* out,
+                                   int ldo, int64_t total) {
   for (int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = e / n;
     const int i = (int)(e - t * n);
-    stf(out + t * ldo + i, a[e] * sigmoidf_(P[t * ldp + g_off + i]));
+    stf(out + t * ldo + i, ldf(a + t * lda + i) * sigmoidf_(P[t * ldp + g_off + i]));
   }
 }
 
@@ -163,21 +164,28 @@ void diff_attn_out(const at::Tensor& a, const at::Tensor& P, int64_t g_off, int6
                                                       out.data_ptr<float>(), ldo);
 }
 
+// a [T, n]: fp32, or rows of out's dtype (also out's own rows: the gate applied in place)
 void sigmoid_gate_mul(const at::Tensor& a, const at::Tensor& P, int64_t g_off, at::Tensor& out) {
-  f32c(a, "a");
   const int ldp = ld_of(P, "P");
   const int64_t T = P.size(0);
   if (T == 0) return;
-  MCHECK(a.dim() == 2 && a.size(0) == T, "a must be [T, n]");
+  MCHECK(a.is_cuda() && a.dim() == 2 && a.size(0) == T && a.stride(1) == 1 &&
+             (a.scalar_type() == at::kFloat || a.scalar_type() == out.scalar_type()),
+         "a must be [T, n] rows, fp32 or of out's dtype");
   const int64_t n = a.size(1);
+  const int lda = (int)a.stride(0);
   cols_ok(P, g_off, n, "gate");
   const int ldo = act_ld_min(out, T, n, "out");
-  if (out.scalar_type() == at::kBFloat16)
-    sigmoid_gate_mul_k<uint16_t><<<grid_for(T * n), 256, 0, stream()>>>(a.data_ptr<float>(), P.data_ptr<float>(), ldp, (int)g_off,
-                                                                        (int)n, (uint16_t*)out.data_ptr(), ldo, T * n);
+  const int grid = grid_for(T * n);
+  if (out.scalar_type() == at::kBFloat16 && a.scalar_type() == at::kFloat)
+    sigmoid_gate_mul_k<float, uint16_t><<<grid, 256, 0, stream()>>>(a.data_ptr<float>(), lda, P.data_ptr<float>(), ldp, (int)g_off,
+                                                                    (int)n, (uint16_t*)out.data_ptr(), ldo, T * n);
+  else if (out.scalar_type() == at::kBFloat16)
+    sigmoid_gate_mul_k<uint16_t, uint16_t><<<grid, 256, 0, stream()>>>((const uint16_t*)a.data_ptr(), lda, P.data_ptr<float>(), ldp,
+                                                                       (int)g_off, (int)n, (uint16_t*)out.data_ptr(), ldo, T * n);
   else
-    sigmoid_gate_mul_k<float><<<grid_for(T * n), 256, 0, stream()>>>(a.data_ptr<float>(), P.data_ptr<float>(), ldp, (int)g_off,
-                                                                     (int)n, out.data_ptr<float>(), ldo, T * n);
+    sigmoid_gate_mul_k<float, float><<<grid, 256, 0, stream()>>>(a.data_ptr<float>(), lda, P.data_ptr<float>(), ldp, (int)g_off,
+                                                                 (int)n, out.data_ptr<float>(), ldo, T * n);
 }
 
 void silu_cols(const at::Tensor& P, int64_t off, int64_t n, at::Tensor& out) {

@@ -68,6 +68,7 @@ _CARDS: List[tuple] = [
   ("tiny-tarepel", 4, "synthetic/tiny-tarepel", "Tiny Tarepel (synthetic)"),
   ("tiny-mogelix", 4, "synthetic/tiny-mogelix", "Tiny Mogelix (synthetic)"),
   ("tiny-nenizen", 5, "synthetic/tiny-nenizen", "Tiny Nenizen (synthetic)"),
+  ("tiny-kopalorn", 4, "synthetic/tiny-kopalorn", "Tiny Kopalorn (synthetic)"),
 ]
 
 model_cards: Dict[str, dict] = {mid: {"layers": n, "repo": {ENGINE: repo}} for mid, n, repo, _ in _CARDS}

@@ -557,11 +557,10 @@ class ShardModel:
       K.kv_pool_update(self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q, inp.ctx_lens,
                        a.pool, inp.max_qlen)
     pool = a.pool if self.kv.kp[j] is not None else 0
-    n = a.heads * a.vdim
-    o = mix[:, :n] if a.gate == "none" else torch.empty(P.shape[0], n, dtype=torch.float32, device=P.device)
+    o = mix[:, :a.heads * a.vdim]
     K.attn_window_pool(q, self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q,
                        inp.ctx_lens, lw.sink, a.scale, a.window, pool, o, max_qlen=inp.max_qlen)
-    if a.gate != "none":  # one sigmoid gate per element, from the mixer's input
+    if a.gate != "none":  # one sigmoid gate per element, from the mixer's input, applied in place
       K.sigmoid_gate_mul(o, P, lw.cols["gate"][0], mix)
 
   def _diff_attn(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:

@@ -623,7 +623,7 @@ def diff_attn_out(a, P, g_off: int, H: int, G: int, lam: float, post: float, eps
 
 
 def sigmoid_gate_mul(a, P, g_off: int, out) -> None:
-  """out[:, :n] = a * sigmoid(P[:, g_off : +n]) for a [T, n]."""
+  """out[:, :n] = a * sigmoid(P[:, g_off : +n]) for a [T, n], fp32 or of out's dtype (out's own rows: in place)."""
   _mix("sigmoid_gate_mul", _gpu(a))(a, P, int(g_off), out)
 
 

@@ -628,7 +628,7 @@ def diff_attn_out(a, P, g_off, H, G, lam, post, eps, out):
 
 def sigmoid_gate_mul(a, P, g_off, out):
   """out[:, :n] = a * sigmoid(P[:, g_off : +n]), n = a's row."""
-  n = a.shape[1]
+  n = a.shape[1]  # (a may be out's own rows)
   out[:, :n] = (a.float() * torch.sigmoid(P[:, g_off:g_off + n].float())).to(out.dtype)
 
 
