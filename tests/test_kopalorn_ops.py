@@ -25,7 +25,7 @@ def close(got, want, tol, what=""):
 
 
 @pytest.mark.parametrize("dev,dtype", RUNS)
-@pytest.mark.parametrize("D", [48, 200, 1100])
+@pytest.mark.parametrize("D", [48, 200, 1100, 3000, 4200])
 def test_layer_norm_add_and_next_norm(dev, dtype, D):
   """x += mult * layer_norm(y) and the next sublayer's input layer_norm(x), biases and all; y rows wider than D."""
   T, eps, mult = 5, 1e-5, 0.3
@@ -127,7 +127,7 @@ def _state_case(H, dv_state, d, dev):
 
 
 @pytest.mark.parametrize("dev,dtype", RUNS)
-@pytest.mark.parametrize("H,d,dv,cap", [(2, 16, 16, 15.0), (3, 24, 40, 2.0), (1, 72, 9, 50.0)])
+@pytest.mark.parametrize("H,d,dv,cap", [(2, 16, 16, 15.0), (3, 24, 40, 2.0), (1, 72, 9, 50.0), (2, 16, 200, 15.0)])
 def test_mlstm_gates_recurrence_and_norm(dev, dtype, H, d, dv, cap):
   """Gates with their cap, the running maximum from zero, decay and input scale, the recurrence with the normaliser as the
   state's last value channel, the stabilised division, the per-head norm, weight and sigmoid gate; states carried over

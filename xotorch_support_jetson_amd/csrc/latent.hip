@@ -560,6 +560,71 @@ __global__ __launch_bounds__(256) void latent_attn_merge_k(const float* __restri
   }
 }
 
+// The same for rows of at most 256 R numbers: a thread keeps its R values of y and of x in registers, so each row is
+// read once (the sums run over registers; the variance still after the mean, as the mean of the squared deviations).
+template <typename AT, int R>
+__global__ __launch_bounds__(256) void sandwich_add_norm_reg_k(float* __restrict__ x, const float* __restrict__ y, int ldy,
+                                                               const float* __restrict__ wb, const float* __restrict__ bb,
+                                                               const float* __restrict__ wn, const float* __restrict__ bn,
+                                                               float mult, float eps, AT* __restrict__ out, int ldo, int D) {
+  __shared__ float red[8];
+  const int64_t t = blockIdx.x;
+  float* xr = x + t * D;
+  float xv[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = threadIdx.x + 256 * r;
+    xv[r] = i < D ? xr[i] : 0.0f;
+  }
+  // (shift, scale) of a row held in registers
+  auto stats = [&](const float* v, bool center, float* mu, float* rs) {
+    float mean = 0.0f;
+    if (center) {
+      float s = 0.0f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) s += v[r];  // (entries past D are zero)
+      mean = block_sum(s, red) / D;
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float c = threadIdx.x + 256 * r < D ? v[r] - mean : 0.0f;
+      ss += c * c;
+    }
+    ss = block_sum(ss, red);
+    *mu = mean;
+    *rs = 1.0f / sqrtf(ss / D + eps);
+  };
+  if (y) {
+    const float* yr = y + t * ldy;
+    float yv[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = threadIdx.x + 256 * r;
+      yv[r] = i < D ? yr[i] : 0.0f;
+    }
+    float mu, rs;
+    stats(yv, bb != nullptr, &mu, &rs);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = threadIdx.x + 256 * r;
+      if (i < D) {
+        xv[r] += mult * ((yv[r] - mu) * rs * wb[i] + (bb ? bb[i] : 0.0f));
+        xr[i] = xv[r];
+      }
+    }
+  }
+  if (wn) {
+    float mu, rs;
+    stats(xv, bn != nullptr, &mu, &rs);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int i = threadIdx.x + 256 * r;
+      if (i < D) stf(out + t * ldo + i, (xv[r] - mu) * rs * wn[i] + (bn ? bn[i] : 0.0f));
+    }
+  }
+}
+
 // ------------------------------------------------------------------ host side
 // XOT_LATT_MFMA=0 keeps prompt portions on the wave-per-tile attention kernel (A/B runs)
 const bool LATT_MFMA = []() { const char* e = getenv("XOT_LATT_MFMA"); return !(e && e[0] == '0'); }();
@@ -602,12 +667,21 @@ void sandwich_add_norm(at::Tensor& x, const c10::optional<at::Tensor>& y, const 
     bf = out->scalar_type() == at::kBFloat16;
   }
   if (!yp && !np) return;
-  if (bf)
-    sandwich_add_norm_k<uint16_t><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, bbp, np, bnp, (float)mult, (float)eps,
-                                                           (uint16_t*)op, ldo, (int)D);
-  else
-    sandwich_add_norm_k<float><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, bbp, np, bnp, (float)mult, (float)eps,
-                                                        (float*)op, ldo, (int)D);
+#define SAN_GO(KERNEL, AT)                                                                                              \
+  KERNEL<<<T, 256, 0, stream()>>>(x.data_ptr<float>(), yp, ldy, bp, bbp, np, bnp, (float)mult, (float)eps, (AT*)op, ldo, \
+                                  (int)D)
+#define SAN_PICK(AT)                                                     \
+  if (D <= 1024) SAN_GO((sandwich_add_norm_reg_k<AT, 4>), AT);           \
+  else if (D <= 2048) SAN_GO((sandwich_add_norm_reg_k<AT, 8>), AT);      \
+  else if (D <= 4096) SAN_GO((sandwich_add_norm_reg_k<AT, 16>), AT);     \
+  else SAN_GO(sandwich_add_norm_k<AT>, AT)
+  if (bf) {
+    SAN_PICK(uint16_t);
+  } else {
+    SAN_PICK(float);
+  }
+#undef SAN_PICK
+#undef SAN_GO
 }
 
 void check_rope(const at::Tensor& pos, const at::Tensor& cos_sin, int64_t T, int64_t rot, int64_t dr) {

@@ -121,6 +121,34 @@ __global__ void gated_group_norm_k(const float* __restrict__ o, const float* __r
   }
 }
 
+// Groups of at most 64 GR values: a wave per (token, group), four groups a workgroup, the group's values in registers.
+template <typename AT, int GR>
+__global__ __launch_bounds__(256) void gated_group_norm_wave_k(const float* __restrict__ o, const float* __restrict__ m,
+                                                               const float* __restrict__ w, const float* __restrict__ P,
+                                                               int ldp, int g_off, int groups, int gs, float eps,
+                                                               AT* __restrict__ out, int ldo) {
+  const int t = blockIdx.x, g = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (g >= groups) return;  // (wave-uniform; no workgroup barrier below)
+  const int extra = m ? 1 : 0;
+  const float* x = o + ((int64_t)t * groups + g) * (gs + extra);
+  float div = 1.0f;
+  if (m) div = 1.0f / (fmaxf(fabsf(x[gs]), expf(-m[(int64_t)t * groups + g])) + 1e-6f);
+  float v[GR];
+  float ss = 0.0f;
+#pragma unroll
+  for (int r = 0; r < GR; ++r) {
+    const int i = lane + 64 * r;
+    v[r] = i < gs ? x[i] * div : 0.0f;
+    ss += v[r] * v[r];
+  }
+  const float k = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+#pragma unroll
+  for (int r = 0; r < GR; ++r) {
+    const int i = lane + 64 * r, c = g * gs + i;
+    if (i < gs) stf(out + (int64_t)t * ldo + c, v[r] * k * w[c] * sigmoidf_(P[(int64_t)t * ldp + g_off + c]));
+  }
+}
+
 // ------------------------------------------------------------------ mean of two normed rows
 __global__ __launch_bounds__(256) void pair_norm_mean_k(const float* __restrict__ y1, int ld1, const float* __restrict__ y2,
                                                         int ld2, const float* __restrict__ w, float eps,
@@ -243,16 +271,26 @@ void gated_group_norm(const at::Tensor& o, const c10::optional<at::Tensor>& m, c
   }
   cols_ok(P, g_off, n, "gate");
   const int ldo = act_ld_min(out, T, n, "out");
+#define GGN_ARGS(AT)                                                                                                      \
+  o.data_ptr<float>(), mp, w.data_ptr<float>(), P.data_ptr<float>(), ldp, (int)g_off, (int)groups, (int)gs, (float)eps, \
+      (AT*)out.data_ptr(), ldo
+  const bool bf = out.scalar_type() == at::kBFloat16;
+  if (gs <= 512 && groups > 1) {  // a wave per group
+    const dim3 grid((unsigned)T, (unsigned)((groups + 3) / 4));
+    if (gs <= 128) {
+      if (bf) gated_group_norm_wave_k<uint16_t, 2><<<grid, 256, 0, stream()>>>(GGN_ARGS(uint16_t));
+      else gated_group_norm_wave_k<float, 2><<<grid, 256, 0, stream()>>>(GGN_ARGS(float));
+    } else {
+      if (bf) gated_group_norm_wave_k<uint16_t, 8><<<grid, 256, 0, stream()>>>(GGN_ARGS(uint16_t));
+      else gated_group_norm_wave_k<float, 8><<<grid, 256, 0, stream()>>>(GGN_ARGS(float));
+    }
+    return;
+  }
   const dim3 grid((unsigned)T, (unsigned)groups);
   const int threads = (int)std::min<int64_t>(256, (gs + 63) / 64 * 64);
-  if (out.scalar_type() == at::kBFloat16)
-    gated_group_norm_k<uint16_t><<<grid, threads, 0, stream()>>>(o.data_ptr<float>(), mp, w.data_ptr<float>(), P.data_ptr<float>(),
-                                                                 ldp, (int)g_off, (int)groups, (int)gs, (float)eps,
-                                                                 (uint16_t*)out.data_ptr(), ldo);
-  else
-    gated_group_norm_k<float><<<grid, threads, 0, stream()>>>(o.data_ptr<float>(), mp, w.data_ptr<float>(), P.data_ptr<float>(),
-                                                              ldp, (int)g_off, (int)groups, (int)gs, (float)eps,
-                                                              out.data_ptr<float>(), ldo);
+  if (bf) gated_group_norm_k<uint16_t><<<grid, threads, 0, stream()>>>(GGN_ARGS(uint16_t));
+  else gated_group_norm_k<float><<<grid, threads, 0, stream()>>>(GGN_ARGS(float));
+#undef GGN_ARGS
 }
 
 void pair_norm_mean(const at::Tensor& y1, const at::Tensor& y2, const at::Tensor& w, double eps, at::Tensor& out) {
