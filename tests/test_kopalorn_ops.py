@@ -75,7 +75,8 @@ def _paged(seqs, slots_of, k_rows, v_rows, G, Gv, d, dv, dev, dtype, pages):
 
 
 @pytest.mark.parametrize("dev,dtype", RUNS)
-@pytest.mark.parametrize("H,G,Gv,d,dv,window", [(8, 4, 2, 16, 24, 11), (4, 2, 1, 32, 64, 70), (2, 2, 2, 48, 48, 0), (16, 2, 1, 8, 8, 64)])
+@pytest.mark.parametrize("H,G,Gv,d,dv,window", [(8, 4, 2, 16, 24, 11), (4, 2, 1, 32, 64, 70), (2, 2, 2, 48, 48, 0), (16, 2, 1, 8, 8, 64),
+                                                  (4, 2, 1, 64, 128, 100), (4, 4, 2, 128, 128, 0), (6, 2, 2, 64, 64, 33)])
 def test_window_attention_with_shared_values(dev, dtype, H, G, Gv, d, dv, window):
   """Key head g reads value head g / (G / Gv); fp32 output beside caches of the activations' dtype; two sequences on
   scrambled pages, a portion of 19 tokens and a single token."""
