@@ -305,7 +305,7 @@ SIZES = [
           layer("mlstm", mlstm(4, 8, 32), None), layer("attention", attention(2, 2, 32, 16, window=5, dims=32), None)],
          width=32, vocab=40, loop=(3, 4, 1)),
   # more experts, groups and chosen experts, eight query heads per kv head, a loop that starts at the first layer
-  config([layer("attention", attention(8, 1, 16, 32, window=40, diff=0.1), moe(8, 48, 9, 0, 8, 3, 2.5)), layer("mlstm", mlstm(2, 16, 16), moe(8, 4, 2, 8, 2, 1))],
+  config([layer("attention", attention(8, 1, 16, 32, window=40, diff=0.1), moe(8, 48, 9, 0, 8, 3, 2.0)), layer("mlstm", mlstm(2, 16, 16), moe(8, 4, 2, 8, 2, 1))],
          width=32, vocab=40, loop=(0, 1, 2)),
 ]
 
