@@ -864,15 +864,10 @@ def build_postln_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWe
     down = get(q + "down")
     lw.act = dev(get(q + "act"))
   else:
-    fb = [("router", get(q + "router"))]
-    down = None
-    if f.shared_ff:
-      fb += [("sh_up", get(q + "shared.up")), ("sh_gate", get(q + "shared.sg").reshape(1, D))]
-      down = get(q + "shared.down")
     lw.router_b = dev(get(q + "router.b"))
-    Fp, Dp = _up(f.ff, 128), _up(D, 128)
-    lw.ex_up_w = dev(torch.stack([_pad2(get(q + f"e{e}.up"), Fp, Dp) for e in range(f.experts)]), dtype)
-    lw.ex_down_w = dev(torch.stack([_pad2(get(q + f"e{e}.down"), Dp, Fp) for e in range(f.experts)]), dtype)
+    _relu2_moe_weights(lw, f, get, q, D, dev, dtype, gate_rows=get(p + "rg2"))
+    lw.norm2, lw.gate2_b = dev(get(p + "norm2")), dev(get(p + "rg2.b"))
+    return lw
   fb.append(("gate", get(p + "rg2")))
   ff_w, lw.ff_cols = _fused_rows(fb, D)
   lw.ff_w = dev(ff_w, dtype)
