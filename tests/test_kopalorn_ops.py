@@ -191,7 +191,7 @@ def test_lightning_recurrence_and_norm(dev, dtype, H, d, dv):
     qkv = torch.empty(T, 2 * nq + nv, device=dev)
     K.silu_cols(P, 0, 2 * nq + nv, qkv)
     o = torch.empty(T, nv, device=dev)
-    K.linear_recurrence(qkv[:, :nq], qkv[:, nq:2 * nq], qkv[:, 2 * nq:], dec.expand(T, H).contiguous(), None, 1.0, S, slots, cuq, o)
+    K.linear_recurrence(qkv[:, :nq], qkv[:, nq:2 * nq], qkv[:, 2 * nq:], dec, None, 1.0, S, slots, cuq, o)
     out = torch.zeros(T, nv, dtype=dtype, device=dev)
     K.gated_group_norm(o, None, t["norm"].to(dev), P, 2 * nq + nv, 1, eps, out)
     for b in range(2):

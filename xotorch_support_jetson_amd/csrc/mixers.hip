@@ -579,7 +579,7 @@ template <int KR, int RS, int MODE>
 __global__ __launch_bounds__(256) void linear_recurrence_k(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
-    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv, int dvin,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv, int dvin, int dstride,
     float* __restrict__ out) {
   constexpr int DP = KR * RS;  // padded key dim
   constexpr bool DELTA = MODE == 1, SCALAR = MODE != 0, NORMCH = MODE == 3;
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
       if (NORMCH && e < TB * COLS && c == dvin && tb + tt < n) pv[j] = 1.0f;
     }
     if (SCALAR && tid < TB && tb + tid < n) {
-      pg0 = decay[(int64_t)(t0 + tb + tid) * H + h];
+      pg0 = decay[(int64_t)(t0 + tb + tid) * dstride + h];  // (dstride 0: one fixed decay per head, decay [H])
       if (DELTA || NORMCH) pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
     }
   };
@@ -992,11 +992,11 @@ void gla_prep(const at::Tensor& P, int64_t a1_off, const at::Tensor& a2, const a
 template <int RS, int MODE>
 void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay,
                 const float* beta, float q_scale, float* state, const int* slots, const int* cu, int H, int G, int d, int dv,
-                int dvin, float* out) {
+                int dvin, int dstride, float* out) {
 #define REC_CASE(DPAD)                                                                                                 \
   case DPAD:                                                                                                           \
     linear_recurrence_k<DPAD / RS, RS, MODE><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, \
-                                                                          state, slots, cu, H, G, d, dv, dvin, out);   \
+                                                                          state, slots, cu, H, G, d, dv, dvin, dstride, out); \
     break;
   switch (KR * RS) {  // padded key dim
     REC_CASE(16)
@@ -1011,7 +1011,8 @@ void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int 
 }
 
 // q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta rule, or
-// without beta: one decay per head and a plain outer-product write) or [T, H d] (per key channel); beta [T, H] (delta
+// without beta: one decay per head and a plain outer-product write; a 1-D [H]: the same decay at every token) or [T, H d]
+// (per key channel); beta [T, H] (delta
 // only; an input scale for a state with a normaliser channel: then v is [T, H (dv - 1)]).  state [slots, H, dv, d] (S^T: key
 // rows contiguous).
 void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& decay,
@@ -1038,10 +1039,12 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   if (beta.has_value()) {
     f32c(*beta, "beta");
     MCHECK(beta->numel() == T * H && decay.numel() == T * H, "delta rule: beta / decay must be [T, H]");
-  } else if (decay.numel() != T * H) {
+  } else if (decay.numel() != T * H && !(decay.dim() == 1 && decay.numel() == H)) {
     MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
   }
-  const bool scalar = !delta && !normch && decay.numel() == T * H;  // one decay per head, q / k shared by H / G heads
+  // one decay per head (and token: [T, H]; or fixed: a 1-D [H]), q / k shared by H / G heads
+  const bool fixed = !delta && !normch && decay.dim() == 1 && decay.numel() == H;
+  const bool scalar = !delta && !normch && (fixed || decay.numel() == T * H);
   int DP = 16;
   while (DP < d) DP *= 2;
   MCHECK(DP <= 256, "linear_recurrence: key dim above 256");
@@ -1054,7 +1057,8 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
 #define REC_GO(R, D)                                                                                                          \
   launch_rec<R, D>(DP / R, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,              \
                    decay.data_ptr<float>(), bp, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),        \
-                   cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, (int)dvin, out.data_ptr<float>())
+                   cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, (int)dvin, fixed ? 0 : (int)H,         \
+                   out.data_ptr<float>())
   if (delta) REC_GO(16, 1); else if (normch) REC_GO(16, 3); else if (scalar) REC_GO(16, 2); else REC_GO(16, 0);
 #undef REC_GO
 }

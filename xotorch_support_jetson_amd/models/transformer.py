@@ -604,7 +604,7 @@ class ShardModel:
     qkv = torch.empty(T, 2 * nq + nv, dtype=torch.float32, device=dev)
     K.silu_cols(P, lw.cols["rq"][0], 2 * nq + nv, qkv)  # (q | k | v are neighbours in the fused projection)
     o = torch.empty(T, nv, dtype=torch.float32, device=dev)
-    K.linear_recurrence(qkv[:, :nq], qkv[:, nq:2 * nq], qkv[:, 2 * nq:], lw.decay.expand(T, H).contiguous(), None, 1.0,
+    K.linear_recurrence(qkv[:, :nq], qkv[:, nq:2 * nq], qkv[:, 2 * nq:], lw.decay, None, 1.0,
                         st.S[j], inp.state_slots, inp.cu_q, o)
     K.gated_group_norm(o, None, lw.rec_norm, P, lw.cols["rg"][0], 1, self.c.rms_norm_eps, mix)
 

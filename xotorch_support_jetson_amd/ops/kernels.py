@@ -490,7 +490,8 @@ def gla_prep(P, a1_off: int, a2, a2_b, tau: float, decay) -> None:
 def linear_recurrence(q, k, v, decay, beta, q_scale: float, state, state_slots, cu_q, out) -> None:
   """Per sequence and value head, token by token on the fp32 state, stored S^T [slots, H, dv, d] (updated in place):
   beta given (delta rule, decay [T, H]):  S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q
-  else (decay [T, H d] per key channel, or [T, H] per head):  S = diag(a) S + k v^T; o = S^T q.   q is scaled by q_scale.
+  else (decay [T, H d] per key channel, [T, H] per head, or a 1-D [H]: fixed per head):  S = diag(a) S + k v^T; o = S^T q.
+  q is scaled by q_scale.
   A state with one value channel more than v has (decay [T, H], beta [T, H] an input scale): S = g S + k (beta [v | 1])^T,
   the last channel being a normaliser n = g n + beta k; out [T, H (dv + 1)] then ends each head with n . q."""
   _mix("linear_recurrence", _gpu(q))(q, k, v, decay, beta, float(q_scale), state, state_slots, cu_q, out)

@@ -320,6 +320,8 @@ def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, o
   _, H, dv, d = state.shape  # stored transposed: S^T [dv, d] per head
   G = q.shape[1] // d
   rep = H // G
+  if decay.dim() == 1 and decay.numel() == H and beta is None:  # one fixed decay per head
+    decay = decay.reshape(1, H).expand(q.shape[0], H)
   norm_ch = v.shape[1] == H * (dv - 1)  # the state's last value channel is a normaliser fed with ones; beta: input scale
   if norm_ch:
     dv -= 1
